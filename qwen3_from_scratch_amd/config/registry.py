@@ -67,9 +67,11 @@ def load_model_config(model_dir):
     with open(path) as fh:
         data = json.load(fh)
     names = data.get("architectures")
+    if names is None and isinstance(data.get("architecture"), str):
+        names = [data["architecture"]]           # some architectures name themselves with one string
     if not names or not isinstance(names, list):
         raise ConfigError(
-            "config.json: 'architectures' must name the model class; known: %s"
+            "config.json: 'architectures' (or 'architecture') must name the model class; known: %s"
             % ", ".join(architectures())
         )
     config_class, _ = lookup_architecture(names[0])

@@ -80,3 +80,25 @@ extern "C" int q3_swiglu(const void* gate_up, void* out, int T, int I, int dtype
   }
   return q3_launch_status();
 }
+
+// out = gelu(x), elementwise in float32, rounded once: kind 0 the exact form
+// 0.5 z (1 + erf(z / sqrt 2)), kind 1 the tanh form 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))).
+__device__ inline float gelu_value(float z, int kind) {
+  if (kind == 0) return 0.5f * z * (1.f + erff(z * 0.70710678118654752f));
+  return 0.5f * z * (1.f + tanhf(0.79788456080286536f * (z + 0.044715f * z * z * z)));
+}
+
+template <typename T>
+__global__ void gelu_kernel(const T* __restrict__ x, T* __restrict__ out, size_t n, int kind) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+    out[i] = from_float<T>(gelu_value(to_float(x[i]), kind));
+}
+
+extern "C" int q3_gelu(const void* x, void* out, long n, int kind, int dtype, hipStream_t stream) {
+  if (n <= 0 || kind < 0 || kind > 1) return Q3_ERR_BAD_ARGUMENT;
+  long blocks = (n + 255) / 256;
+  if (blocks > 8192) blocks = 8192;
+  Q3_DISPATCH_DTYPE(dtype, TT, hipLaunchKernelGGL(gelu_kernel<TT>, dim3((unsigned)blocks), dim3(256), 0, stream,
+                                                  (const TT*)x, (TT*)out, (size_t)n, kind));
+  return q3_launch_status();
+}

@@ -1,0 +1,251 @@
+// A routed feed-forward: a float32 router with softmax scores and a choice of the `top` best
+// experts per token, the (token, choice) pairs put in the order of their experts, the experts'
+// products over those runs of rows, and the weighted sum per token.
+#include "common.h"
+
+#include <math.h>
+
+__device__ inline float moe_gelu(float z, int kind) {
+  if (kind == 0) return 0.5f * z * (1.f + erff(z * 0.70710678118654752f));
+  return 0.5f * z * (1.f + tanhf(0.79788456080286536f * (z + 0.044715f * z * z * z)));
+}
+
+// ---------------------------------------------------------------------------
+// The router. One wavefront per token: z_e = router[e] . h (float32 sums over bfloat16 or float32
+// numbers), s = softmax(z) over all E experts, then `top` times the largest remaining score (the
+// lowest index among equals); weight_k = s_k / (sum of the chosen s + 1e-20).
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ h, const T* __restrict__ router,
+                                                        int n_tokens, int width, int E, int top,
+                                                        int* __restrict__ chosen, float* __restrict__ weights) {
+  extern __shared__ float smem[];
+  const int wave = threadIdx.x / Q3_WAVE, lane = threadIdx.x % Q3_WAVE;
+  const int t = blockIdx.x * (blockDim.x / Q3_WAVE) + wave;
+  if (t >= n_tokens) return;
+  float* z = smem + (size_t)wave * (E + top);     // the wavefront's scores, then the chosen ones
+  float* picked = z + E;
+  const T* x = h + (size_t)t * width;
+  // every lane holds every sum after the butterfly and writes the same number to the same place,
+  // so nothing here waits for another lane's write
+  for (int e = 0; e < E; ++e) {
+    const T* w = router + (size_t)e * width;
+    float acc = 0.f;
+    for (int j = lane; j < width; j += Q3_WAVE) acc += to_float(x[j]) * to_float(w[j]);
+    z[e] = wave_sum(acc);
+  }
+  __builtin_amdgcn_wave_barrier();
+  float biggest = -INFINITY;
+  for (int e = lane; e < E; e += Q3_WAVE) biggest = fmaxf(biggest, z[e]);
+  biggest = wave_max(biggest);
+  float total = 0.f;
+  for (int e = lane; e < E; e += Q3_WAVE) {
+    const float p = expf(z[e] - biggest);
+    z[e] = p;
+    total += p;
+  }
+  total = wave_sum(total);
+  __builtin_amdgcn_wave_barrier();
+  float picked_sum = 0.f;
+  for (int k = 0; k < top; ++k) {
+    float best = -1.f;
+    int at = 0x7fffffff;
+    for (int e = lane; e < E; e += Q3_WAVE) {
+      const float p = z[e];
+      if (p > best) {
+        best = p;
+        at = e;
+      }
+    }
+#pragma unroll
+    for (int off = Q3_WAVE / 2; off > 0; off >>= 1) {
+      const float ob = __shfl_xor(best, off, Q3_WAVE);
+      const int oa = __shfl_xor(at, off, Q3_WAVE);
+      if (ob > best || (ob == best && oa < at)) {
+        best = ob;
+        at = oa;
+      }
+    }
+    const float score = best / total;
+    picked_sum += score;
+    __builtin_amdgcn_wave_barrier();
+    picked[k] = score;
+    z[at] = -2.f;               // taken
+    if (lane == 0) chosen[(size_t)t * top + k] = at;
+    __builtin_amdgcn_wave_barrier();
+  }
+  const float inv = 1.f / (picked_sum + 1e-20f);
+  for (int k = lane; k < top; k += Q3_WAVE) weights[(size_t)t * top + k] = picked[k] * inv;
+}
+
+// ---------------------------------------------------------------------------
+// Pairs in the order of their experts. One block. `chosen` (P) names each pair's expert.
+//   offsets[e] .. offsets[e+1]: the slots of expert e;  pair_of_slot[slot] = pair;
+//   slot_of_pair[pair] = slot;  tiles of `tile_rows` slots that never cross an expert's end:
+//   tile_expert[i], tile_first[i] (first slot), n_tiles[0].
+// Which slot of its expert's run a pair gets depends on the order in which threads arrive; a
+// row's result does not depend on its slot.
+// ---------------------------------------------------------------------------
+__global__ void moe_align_kernel(const int* __restrict__ chosen, int P, int E, int tile_rows,
+                                 int* __restrict__ offsets, int* __restrict__ pair_of_slot,
+                                 int* __restrict__ slot_of_pair, int* __restrict__ tile_expert,
+                                 int* __restrict__ tile_first, int* __restrict__ n_tiles) {
+  extern __shared__ int counts[];   // [E] counts, then [E] cursors
+  int* cursor = counts + E;
+  for (int e = threadIdx.x; e < E; e += blockDim.x) counts[e] = 0;
+  __syncthreads();
+  for (int p = threadIdx.x; p < P; p += blockDim.x) {
+    const int e = chosen[p];
+    if (e >= 0 && e < E) atomicAdd(&counts[e], 1);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int at = 0, tiles = 0;
+    for (int e = 0; e < E; ++e) {
+      offsets[e] = at;
+      cursor[e] = at;
+      for (int r = 0; r < counts[e]; r += tile_rows) {
+        tile_expert[tiles] = e;
+        tile_first[tiles] = at + r;
+        ++tiles;
+      }
+      at += counts[e];
+    }
+    offsets[E] = at;
+    n_tiles[0] = tiles;
+  }
+  __syncthreads();
+  for (int p = threadIdx.x; p < P; p += blockDim.x) {
+    const int e = chosen[p];
+    if (e >= 0 && e < E) {
+      const int slot = atomicAdd(&cursor[e], 1);
+      pair_of_slot[slot] = p;
+      slot_of_pair[p] = slot;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// The experts' products over the sorted slots, float32 multiply-adds, any sizes:
+//   out[slot, n] = act(sum_k x[src(slot), k] * w[e, n, k]),  e the expert of the slot's tile,
+//   src(slot) = pair_of_slot[slot] / pairs_per_row if `gather` else slot.
+// A block: one tile of 16 slots, 64 output columns; x and w pass shared memory in slices of 32 k.
+// ---------------------------------------------------------------------------
+#define MOE_BM 16
+#define MOE_BN 64
+#define MOE_BK 32
+
+template <typename T>
+__global__ __launch_bounds__(256) void moe_linear_kernel(const T* __restrict__ x, const int* __restrict__ pair_of_slot,
+                                                         int gather, int pairs_per_row, const T* __restrict__ w,
+                                                         T* __restrict__ out, const int* __restrict__ tile_expert,
+                                                         const int* __restrict__ tile_first,
+                                                         const int* __restrict__ offsets,
+                                                         const int* __restrict__ n_tiles, int N, int K, int act) {
+  __shared__ float xs[MOE_BM][MOE_BK + 1];
+  __shared__ float ws[MOE_BN][MOE_BK + 1];
+  __shared__ int src_row[MOE_BM];
+  const int tile = blockIdx.x;
+  if (tile >= n_tiles[0]) return;
+  const int e = tile_expert[tile];
+  const int first = tile_first[tile];
+  const int rows = min(MOE_BM, offsets[e + 1] - first);
+  const int n0 = blockIdx.y * MOE_BN;
+  const int t = threadIdx.x;
+  if (t < MOE_BM) src_row[t] = t < rows ? (gather ? pair_of_slot[first + t] / pairs_per_row : first + t) : -1;
+  __syncthreads();
+  const int r = t >> 4, c = t & 15;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  const T* we = w + (size_t)e * N * K;
+  for (int k0 = 0; k0 < K; k0 += MOE_BK) {
+    for (int idx = t; idx < MOE_BM * MOE_BK; idx += 256) {
+      const int m = idx / MOE_BK, kk = idx - m * MOE_BK;
+      const int s = src_row[m];
+      xs[m][kk] = (s >= 0 && k0 + kk < K) ? to_float(x[(size_t)s * K + k0 + kk]) : 0.f;
+    }
+    for (int idx = t; idx < MOE_BN * MOE_BK; idx += 256) {
+      const int n = idx / MOE_BK, kk = idx - n * MOE_BK;
+      ws[n][kk] = (n0 + n < N && k0 + kk < K) ? to_float(we[(size_t)(n0 + n) * K + k0 + kk]) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < MOE_BK; ++kk) {
+      const float a = xs[r][kk];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[j] += a * ws[c + 16 * j][kk];
+    }
+    __syncthreads();
+  }
+  if (r < rows) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = n0 + c + 16 * j;
+      if (n < N) out[(size_t)(first + r) * N + n] = from_float<T>(act >= 0 ? moe_gelu(acc[j], act) : acc[j]);
+    }
+  }
+}
+
+// out[t, :] = sum_k weights[t, k] * y[slot_of_pair[t * top + k], :] (+ shared[t, :]), float32 sums in
+// the order k = 0, 1, ..., the shared expert last; rounded once.
+template <typename T>
+__global__ void moe_combine_kernel(const T* __restrict__ y, const int* __restrict__ slot_of_pair,
+                                   const float* __restrict__ weights, const T* __restrict__ shared,
+                                   T* __restrict__ out, int width, int top) {
+  const int t = blockIdx.x;
+  for (int j = threadIdx.x; j < width; j += blockDim.x) {
+    float acc = 0.f;
+    for (int k = 0; k < top; ++k) {
+      const int slot = slot_of_pair[(size_t)t * top + k];
+      acc += weights[(size_t)t * top + k] * to_float(y[(size_t)slot * width + j]);
+    }
+    if (shared) acc += to_float(shared[(size_t)t * width + j]);
+    out[(size_t)t * width + j] = from_float<T>(acc);
+  }
+}
+
+extern "C" int q3_moe_route(const void* h, const void* router, int n_tokens, int width, int E, int top, int* chosen,
+                            float* weights, int dtype, hipStream_t stream) {
+  if (n_tokens <= 0 || width <= 0 || E <= 0 || top <= 0 || top > E || E > 4096) return Q3_ERR_BAD_ARGUMENT;
+  const int waves = 4;
+  const size_t smem = (size_t)waves * (E + top) * sizeof(float);
+  Q3_DISPATCH_DTYPE(dtype, TT,
+                    hipLaunchKernelGGL(moe_route_kernel<TT>, dim3((n_tokens + waves - 1) / waves), dim3(waves * Q3_WAVE),
+                                       smem, stream, (const TT*)h, (const TT*)router, n_tokens, width, E, top, chosen,
+                                       weights));
+  return q3_launch_status();
+}
+
+extern "C" int q3_moe_tile_rows() { return MOE_BM; }
+
+extern "C" int q3_moe_align(const int* chosen, int P, int E, int* offsets, int* pair_of_slot, int* slot_of_pair,
+                            int* tile_expert, int* tile_first, int* n_tiles, hipStream_t stream) {
+  if (P <= 0 || E <= 0 || E > 4096) return Q3_ERR_BAD_ARGUMENT;
+  hipLaunchKernelGGL(moe_align_kernel, dim3(1), dim3(1024), (size_t)2 * E * sizeof(int), stream, chosen, P, E, MOE_BM,
+                     offsets, pair_of_slot, slot_of_pair, tile_expert, tile_first, n_tiles);
+  return q3_launch_status();
+}
+
+extern "C" int q3_moe_linear(const void* x, const int* pair_of_slot, int gather, int pairs_per_row, const void* w,
+                             void* out, const int* tile_expert, const int* tile_first, const int* offsets,
+                             const int* n_tiles, int max_tiles, int N, int K, int act, int dtype,
+                             hipStream_t stream) {
+  if (max_tiles <= 0 || N <= 0 || K <= 0 || pairs_per_row <= 0 || act < -1 || act > 1) return Q3_ERR_BAD_ARGUMENT;
+  const dim3 grid(max_tiles, (N + MOE_BN - 1) / MOE_BN);
+  if (grid.y > 65535) return Q3_ERR_UNSUPPORTED;
+  Q3_DISPATCH_DTYPE(dtype, TT,
+                    hipLaunchKernelGGL(moe_linear_kernel<TT>, grid, dim3(256), 0, stream, (const TT*)x, pair_of_slot,
+                                       gather, pairs_per_row, (const TT*)w, (TT*)out, tile_expert, tile_first, offsets,
+                                       n_tiles, N, K, act));
+  return q3_launch_status();
+}
+
+extern "C" int q3_moe_combine(const void* y, const int* slot_of_pair, const float* weights, const void* shared,
+                              void* out, int n_tokens, int width, int top, int dtype, hipStream_t stream) {
+  if (n_tokens <= 0 || width <= 0 || top <= 0) return Q3_ERR_BAD_ARGUMENT;
+  int threads = 64;
+  while (threads < 256 && threads < width) threads *= 2;
+  Q3_DISPATCH_DTYPE(dtype, TT,
+                    hipLaunchKernelGGL(moe_combine_kernel<TT>, dim3(n_tokens), dim3(threads), 0, stream, (const TT*)y,
+                                       slot_of_pair, weights, (const TT*)shared, (TT*)out, width, top));
+  return q3_launch_status();
+}

@@ -137,3 +137,76 @@ extern "C" int q3_rmsnorm(float* x, const void* delta, const void* weight, const
       x, delta, weight, rows, out, n_out, n_src, H, eps, write_back, stream))));
   return Q3_ERR_BAD_ARGUMENT;
 }
+
+// The norm behind a block that also normalises what its parts return, and behind a vector that a
+// model adds to the stream between two layers. One block per output row r (source row s):
+//   a = delta[s]                      the part's result, if there is one
+//   a = a * rsqrt(mean(a^2) + delta_eps) * delta_weight      if delta_weight is given
+//   v = x[s] + a + bias;  if write_back: x[s] = v
+//   out[r] = v * rsqrt(mean(v^2) + eps) * weight             if out is given
+// All float32; the addend is never rounded on its way into the stream. The row lives in shared
+// memory between the passes (`H` floats).
+template <typename T, typename W>
+__global__ void rmsnorm_addend_kernel(float* __restrict__ x, const T* __restrict__ delta,
+                                      const W* __restrict__ delta_weight, float delta_eps,
+                                      const float* __restrict__ bias, const W* __restrict__ weight,
+                                      const int* __restrict__ rows, T* __restrict__ out, int H, int n_src,
+                                      float eps, int write_back) {
+  extern __shared__ float smem[];
+  float* red = smem;
+  float* row = smem + 32;
+  const int r = blockIdx.x;
+  int s = rows ? rows[r] : r;
+  if (s < 0 || s >= n_src) s = 0;
+  float* xs = x + (size_t)s * H;
+  const T* ds = delta ? delta + (size_t)s * H : nullptr;
+  float dscale = 1.f;
+  if (ds && delta_weight) {
+    float acc = 0.f;
+    for (int j = threadIdx.x; j < H; j += blockDim.x) {
+      const float a = to_float(ds[j]);
+      row[j] = a;
+      acc += a * a;
+    }
+    dscale = rsqrtf(block_sum(acc, red) / (float)H + delta_eps);
+  }
+  float acc = 0.f;
+  for (int j = threadIdx.x; j < H; j += blockDim.x) {
+    float v = xs[j];
+    if (ds) v += delta_weight ? row[j] * dscale * to_float(delta_weight[j]) : to_float(ds[j]);
+    if (bias) v += bias[j];
+    row[j] = v;
+    acc += v * v;
+  }
+  const float total = block_sum(acc, red);
+  const float scale = rsqrtf(total / (float)H + eps);
+  for (int j = threadIdx.x; j < H; j += blockDim.x) {
+    const float v = row[j];
+    if (write_back) xs[j] = v;
+    if (out) out[(size_t)r * H + j] = from_float<T>(v * scale * to_float(weight[j]));
+  }
+}
+
+extern "C" int q3_rmsnorm_addend(float* x, const void* delta, const void* delta_weight, float delta_eps,
+                                 const float* bias, const void* weight, const int* rows, void* out, int n_out,
+                                 int n_src, int H, float eps, int act_dtype, int w_dtype, int write_back,
+                                 hipStream_t stream) {
+  if (n_out <= 0 || n_src <= 0 || H <= 0 || H > 36000) return Q3_ERR_BAD_ARGUMENT;
+  if (write_back && rows) return Q3_ERR_BAD_ARGUMENT;
+  if (out && !weight) return Q3_ERR_BAD_ARGUMENT;
+  int threads = 64;
+  while (threads < 1024 && threads * 4 < H) threads *= 2;
+  const size_t smem = (size_t)(32 + H) * sizeof(float);
+  Q3_DISPATCH_DTYPE(act_dtype, TT, Q3_DISPATCH_DTYPE(w_dtype, WW, {
+    if (smem > 48 * 1024) {
+      hipError_t e = hipFuncSetAttribute((const void*)rmsnorm_addend_kernel<TT, WW>,
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+      if (e != hipSuccess) return (int)e;
+    }
+    hipLaunchKernelGGL((rmsnorm_addend_kernel<TT, WW>), dim3(n_out), dim3(threads), smem, stream, x,
+                       (const TT*)delta, (const WW*)delta_weight, delta_eps, bias, (const WW*)weight, rows,
+                       (TT*)out, H, n_src, eps, write_back);
+    return q3_launch_status();
+  }));
+  return Q3_ERR_BAD_ARGUMENT;
+}

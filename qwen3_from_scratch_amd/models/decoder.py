@@ -49,9 +49,12 @@ class DecoderModel:
         self.layers = [_Layer(ls, precision, device,
                               self.position if ls.position is None else self.layer_positions[ls.position])
                        for ls in spec.layers]
+        self.pass_vectors = (build_part(spec.pass_vectors, spec.pass_vectors_prefix, precision, device)
+                             if spec.pass_vectors is not None else None)
         self.final_norm = build_part(spec.final_norm, spec.final_norm_prefix, precision, device)
         self.head = build_part(spec.head, spec.head_prefix, precision, device)
         # each run-order entry that owns a cache gets a plane; readers point at the owner's
+        self.observer = None      # called with (run-order entry, stream, what it still lacks) behind every layer
         self.plane_of_step = []
         self.plane_needs = []
         for i, step in enumerate(spec.order):
@@ -69,6 +72,8 @@ class DecoderModel:
         yield from self.layer_positions.values()
         for layer in self.layers:
             yield from layer.parts()
+        if self.pass_vectors is not None:
+            yield self.pass_vectors
         yield self.final_norm
         yield self.head
 
@@ -136,8 +141,14 @@ class DecoderModel:
             view = cache.view(self.plane_of_step[i], writes=step.reads_cache_of is None)
             # the norm at the next block's entry, if that block can take over its division
             entry = getattr(self.layers[order[i + 1].layer].block, "entry_norm", None) if i + 1 < len(order) else None
+            if entry is not None and order[i + 1].enters is not None:
+                entry = None                      # a pass's vector still has to join the stream in between
+            if step.enters is not None:
+                pending = self.pass_vectors.join(pending, step.enters)
             x, pending = self.layers[step.layer].block.forward(x, pending, batch, view,
                                                                next_norm=entry() if entry else None)
+            if self.observer is not None:
+                self.observer(i, x, pending)
         h = self.final_norm.forward(x, delta=pending, rows=batch.logits_rows)
         return self.head.forward(h)
 

@@ -62,10 +62,14 @@ class RunStep:
     """One entry of the run order. `layer` indexes ModelSpec.layers (a layer
     may be named by several entries: its weights are shared, each entry has a
     cache of its own). `reads_cache_of` names an earlier entry of the run order
-    whose cache this entry's mixer reads without writing; None = its own."""
+    whose cache this entry's mixer reads without writing; None = its own.
+    `enters`: the number of the pass that begins with this entry, for a model that goes through
+    a run of its layers several times (`ModelSpec.pass_vectors`): that pass's vector is added
+    to the residual stream right before the entry's layer."""
 
     layer: int
     reads_cache_of: int = None
+    enters: int = None
 
 
 @dataclass(frozen=True)
@@ -82,9 +86,13 @@ class ModelSpec:
     head: PartSpec
     head_prefix: str = ""
     ignorable_tensors: tuple = ()
+    pass_vectors: PartSpec = None          # a part with `join(pending, number)`, for entries that say `enters`
+    pass_vectors_prefix: str = ""
 
     def __post_init__(self):
         for i, step in enumerate(self.order):
+            if step.enters is not None and self.pass_vectors is None:
+                raise ValueError("run order entry %d begins a pass, but the model has no pass vectors" % i)
             if not (0 <= step.layer < len(self.layers)):
                 raise ValueError("run order entry %d names layer %d of %d" % (i, step.layer, len(self.layers)))
             if step.reads_cache_of is not None:
@@ -114,4 +122,5 @@ def with_components(spec, resolved):
         block=swap(ls.block), position=swap(ls.position))
         for ls in spec.layers)
     return dataclasses.replace(spec, embedding=swap(spec.embedding), position=swap(spec.position), layers=layers,
-                               final_norm=swap(spec.final_norm), head=swap(spec.head))
+                               final_norm=swap(spec.final_norm), head=swap(spec.head),
+                               pass_vectors=swap(spec.pass_vectors))

@@ -24,12 +24,20 @@ __all__ = [
     "loaded_libraries",
     "embed_rows",
     "rmsnorm",
+    "rmsnorm_addend",
     "rope_table",
     "qk_norm_rope_store",
     "paged_attention",
     "decode_attention",
     "decode_attention_takes",
     "swiglu",
+    "gelu",
+    "latent_prepare",
+    "headwise_linear",
+    "rotate_heads",
+    "latent_attention",
+    "moe_route",
+    "moe_experts",
     "linear",
     "linear_plain",
     "linear_swiglu",
@@ -286,6 +294,230 @@ def rmsnorm(x, weight, eps, out_dtype, delta=None, rows=None, write_back=True, o
             _ptr(x), _ptr(delta), _ptr(weight), _ptr(rows), _ptr(out), n_out, T, H,
             ctypes.c_float(eps), _DT[out_dtype], _DT[weight.dtype],
             1 if (write_back and delta is not None) else 0, _stream()), "rmsnorm")
+    return out
+
+
+def rmsnorm_addend(x, weight, eps, out_dtype, delta=None, delta_weight=None, delta_eps=0.0, bias=None, rows=None,
+                   write_back=True, out=None):
+    """The norm of the float32 stream behind an addend that is itself normalised first, and behind
+    a vector added to every row, all in float32 and in one kernel:
+
+    a = delta[s] * rsqrt(mean(delta[s]^2) + delta_eps) * delta_weight (or delta[s] as it is without
+    `delta_weight`, or nothing); v = x[s] + a + bias; x[s] = v if `write_back`;
+    out[r] = v * rsqrt(mean(v^2) + eps) * weight, rounded once to `out_dtype`. With `weight` None
+    only the stream is brought up to date and None is returned. `delta` (T, H) has the activation
+    dtype, `bias` (H,) is float32, `rows` as in `rmsnorm`."""
+    _dev(x, weight, delta, delta_weight, bias, rows, out)
+    _need(x.dim() == 2 and x.dtype == torch.float32, "x must be float32 (T, H)")
+    T, H = x.shape
+    _need(out_dtype in _DT, "out_dtype must be bfloat16 or float32")
+    w_dtype = None
+    for w in (weight, delta_weight):
+        if w is not None:
+            _need(w.shape == (H,) and w.dtype in _DT and w_dtype in (None, w.dtype), "norm weights must be (H,) of one dtype")
+            w_dtype = w.dtype
+    if delta is not None:
+        _need(delta.shape == (T, H) and delta.dtype == out_dtype, "delta must be (T, H) of the activation dtype")
+    _need(delta is not None or delta_weight is None, "a delta weight needs a delta")
+    if bias is not None:
+        _need(bias.shape == (H,) and bias.dtype == torch.float32, "bias must be float32 (H,)")
+    n_out = T
+    if rows is not None:
+        _need(rows.dtype == torch.int32 and rows.dim() == 1, "rows must be int32 (R,)")
+        n_out = rows.shape[0]
+    if weight is None:
+        _need(out is None and rows is None, "without a weight there is no output")
+    elif out is None:
+        out = torch.empty((n_out, H), dtype=out_dtype, device=x.device)
+    if out is not None:
+        _need(out.shape == (n_out, H) and out.dtype == out_dtype, "out must be (rows, H) of out_dtype")
+    write = 1 if (write_back and rows is None and (delta is not None or bias is not None)) else 0
+    if n_out:
+        _check(library("norm").q3_rmsnorm_addend(
+            _ptr(x), _ptr(delta), _ptr(delta_weight), ctypes.c_float(delta_eps), _ptr(bias), _ptr(weight), _ptr(rows),
+            _ptr(out), n_out, T, H, ctypes.c_float(eps), _DT[out_dtype], _DT[w_dtype or torch.float32], write, _stream()),
+            "rmsnorm_addend")
+    return out
+
+
+def gelu(x, kind="erf", out=None):
+    """gelu(x) elementwise in float32, rounded once. `kind`: "erf" for 0.5 z (1 + erf(z / sqrt 2)),
+    "tanh" for 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3)))."""
+    _dev(x, out)
+    _need(x.dtype in _DT and kind in GELU_KINDS, "x bfloat16 or float32; kind erf or tanh")
+    if out is None:
+        out = torch.empty_like(x)
+    _need(out.shape == x.shape and out.dtype == x.dtype, "out must be like x")
+    if x.numel():
+        _check(library("elementwise").q3_gelu(_ptr(x), _ptr(out), ctypes.c_long(x.numel()), GELU_KINDS[kind],
+                                              _DT[x.dtype], _stream()), "gelu")
+    return out
+
+
+GELU_KINDS = {"erf": 0, "tanh": 1}
+
+
+def latent_prepare(down, q_rank, kv_rank, rot_dim, q_weight, kv_weight, eps, inv_freq, rot_factor, positions, seq_index,
+                   block_table=None, cache=None):
+    """The narrow vectors of latent attention from their joint down-projection, in float32:
+
+    down (T, q_rank + kv_rank + rot_dim) holds [query latent | key/value latent | key part to be
+    rotated]. Returns the normalised query latent (T, q_rank) (`q_weight`, `eps`), and writes
+    [normalised key/value latent (`kv_weight`) | rotated key part] as the token's row of `cache`
+    (pages, page, kv_rank + rot_dim) at page block_table[seq_index[t], position // page]; entries
+    below zero are skipped, nothing is written without a cache. The rotation turns the pairs
+    (2i, 2i + 1), i < len(inv_freq), by float32(position) * inv_freq[i], with cos and sin
+    multiplied by `rot_factor`; what lies beyond the pairs passes."""
+    _dev(down, q_weight, kv_weight, inv_freq, positions, seq_index, block_table, cache)
+    R = q_rank + kv_rank + rot_dim
+    _need(down.dim() == 2 and down.shape[1] == R and down.dtype in _DT, "down must be (T, q_rank + kv_rank + rot_dim)")
+    T = down.shape[0]
+    _need(q_weight.shape == (q_rank,) and kv_weight.shape == (kv_rank,) and q_weight.dtype in _DT
+          and kv_weight.dtype == q_weight.dtype, "norm weights (q_rank,) and (kv_rank,) of one dtype")
+    _need(inv_freq.dtype == torch.float32 and inv_freq.dim() == 1 and 2 * inv_freq.shape[0] <= rot_dim,
+          "inv_freq float32, at most rot_dim / 2 pairs")
+    for t in (positions, seq_index):
+        _need(t.dtype == torch.int32 and t.shape == (T,), "positions and seq_index must be int32 (T,)")
+    page = pages = stride = rows = 0
+    if cache is not None:
+        _need(block_table is not None and block_table.dim() == 2 and block_table.dtype == torch.int32,
+              "a cache needs an int32 block table (B, W)")
+        _need(cache.dim() == 3 and cache.shape[2] == kv_rank + rot_dim and cache.dtype == down.dtype,
+              "cache must be (pages, page, kv_rank + rot_dim) of the activation dtype")
+        pages, page = cache.shape[0], cache.shape[1]
+        rows, stride = block_table.shape
+    cq = torch.empty((T, q_rank), dtype=down.dtype, device=down.device)
+    if T:
+        _check(library("latent").q3_latent_prepare(
+            _ptr(down), T, q_rank, kv_rank, rot_dim, _ptr(q_weight), _ptr(kv_weight), _DT[q_weight.dtype],
+            ctypes.c_float(eps), _ptr(inv_freq), inv_freq.shape[0], ctypes.c_float(rot_factor), _ptr(positions),
+            _ptr(seq_index), _ptr(block_table), stride, rows, _ptr(cache), page, pages, _ptr(cq), _DT[down.dtype],
+            _stream()), "latent_prepare")
+    return cq
+
+
+def headwise_linear(x, weight, out=None):
+    """out[t, h, :] = weight[h]^T x[t, h, :]: x (T, H, I) seen through strides (its last axis
+    contiguous), weight (H, I, O) contiguous, out (T, H, O) likewise seen through strides; float32
+    sums in the order of I."""
+    _dev(weight)
+    _need(x.is_cuda and x.dim() == 3 and x.stride(2) == 1 and weight.dim() == 3 and x.dtype in _DT
+          and weight.dtype == x.dtype, "x (T, H, I) with a contiguous last axis, weight (H, I, O), one dtype")
+    T, H, I = x.shape
+    O = weight.shape[2]
+    _need(weight.shape == (H, I, O), "weight must be (H, I, O)")
+    if out is None:
+        out = torch.empty((T, H, O), dtype=x.dtype, device=x.device)
+    _need(out.is_cuda and out.shape == (T, H, O) and out.stride(2) == 1 and out.dtype == x.dtype, "out must be (T, H, O)")
+    if T:
+        _check(library("latent").q3_headwise_linear(
+            _ptr(x), ctypes.c_long(x.stride(0)), x.stride(1), _ptr(weight), _ptr(out), ctypes.c_long(out.stride(0)),
+            out.stride(1), T, H, I, O, _DT[x.dtype], _stream()), "headwise_linear")
+    return out
+
+
+def rotate_heads(x, out, inv_freq, rot_factor, positions):
+    """out[t, h, :] = x[t, h, :] with its pairs (2i, 2i + 1), i < len(inv_freq), turned by
+    float32(positions[t]) * inv_freq[i] (cos and sin times `rot_factor`), the rest copied; x and
+    out (T, H, n) seen through strides."""
+    _dev(inv_freq, positions)
+    _need(x.is_cuda and out.is_cuda and x.dim() == 3 and out.shape == x.shape and x.stride(2) == 1
+          and out.stride(2) == 1 and x.dtype in _DT and out.dtype == x.dtype, "x and out (T, H, n) of one dtype")
+    T, H, n = x.shape
+    _need(inv_freq.dtype == torch.float32 and inv_freq.dim() == 1 and 2 * inv_freq.shape[0] <= n, "inv_freq float32")
+    _need(positions.dtype == torch.int32 and positions.shape == (T,), "positions int32 (T,)")
+    if T:
+        _check(library("latent").q3_rotate_heads(
+            _ptr(x), ctypes.c_long(x.stride(0)), x.stride(1), _ptr(out), ctypes.c_long(out.stride(0)), out.stride(1),
+            T, H, n, inv_freq.shape[0], _ptr(inv_freq), ctypes.c_float(rot_factor), _ptr(positions), _DT[x.dtype],
+            _stream()), "rotate_heads")
+    return out
+
+
+def latent_attention(q, cache, value_dim, block_table, cu_seqlens_q, kv_lens, max_q_len, scale, window=0):
+    """Causal softmax attention of every head's query rows over one shared sequence of cached rows.
+
+    q (T, H, Dk) contiguous; cache (pages, page, Dk): the row of sequence b's position j lies in
+    page block_table[b, j // page]; a row is the key in full and the value in its first
+    `value_dim` numbers. The query of token i of sequence b (position kv_lens[b] - q_len + i) sees
+    positions j <= its own and, with window > 0, only those fewer than `window` behind it.
+    Returns (T, H, value_dim). Float32 scores, statistics and sums."""
+    _dev(q, cache, block_table, cu_seqlens_q, kv_lens)
+    _need(q.dim() == 3 and q.dtype in _DT and cache.dim() == 3 and cache.dtype == q.dtype
+          and cache.shape[2] == q.shape[2], "q (T, H, Dk) and cache (pages, page, Dk) of one dtype")
+    T, H, Dk = q.shape
+    B = kv_lens.shape[0]
+    _need(0 < value_dim <= Dk, "the value is a leading part of the cached row")
+    _need(cu_seqlens_q.dtype == torch.int32 and cu_seqlens_q.shape == (B + 1,) and kv_lens.dtype == torch.int32,
+          "cu_seqlens_q int32 (B + 1,), kv_lens int32 (B,)")
+    _need(block_table.dim() == 2 and block_table.dtype == torch.int32 and block_table.shape[0] >= B,
+          "block_table must be int32 (B, W)")
+    out = torch.empty((T, H, value_dim), dtype=q.dtype, device=q.device)
+    if T and B:
+        _check(library("latent").q3_latent_attention(
+            _ptr(q), _ptr(out), _ptr(cache), cache.shape[0], _ptr(block_table), block_table.shape[1],
+            _ptr(cu_seqlens_q), _ptr(kv_lens), B, H, Dk, value_dim, cache.shape[1], ctypes.c_float(scale), int(window),
+            int(max_q_len), _DT[q.dtype], _stream()), "latent_attention")
+    return out
+
+
+def moe_route(h, router, top):
+    """Per token the `top` experts with the largest softmax scores and their weights: h (T, width),
+    router (E, width) of h's dtype; logits and scores float32. Returns chosen int32 (T, top), in
+    the order of falling score (the lowest index among equals), and weights float32 (T, top) =
+    score / (sum of the chosen scores + 1e-20)."""
+    _dev(h, router)
+    _need(h.dim() == 2 and router.dim() == 2 and h.shape[1] == router.shape[1] and h.dtype in _DT
+          and router.dtype == h.dtype, "h (T, width) and router (E, width) of one dtype")
+    T, E = h.shape[0], router.shape[0]
+    _need(1 <= top <= E, "top must lie in 1..E")
+    chosen = torch.empty((T, top), dtype=torch.int32, device=h.device)
+    weights = torch.empty((T, top), dtype=torch.float32, device=h.device)
+    if T:
+        _check(library("moe").q3_moe_route(_ptr(h), _ptr(router), T, h.shape[1], E, top, _ptr(chosen), _ptr(weights),
+                                           _DT[h.dtype], _stream()), "moe_route")
+    return chosen, weights
+
+
+def moe_experts(h, chosen, weights, up, down, shared=None, activation="erf"):
+    """sum_k weights[t, k] * down[e] act(up[e] h[t]), e = chosen[t, k], plus `shared[t]` if given:
+    h (T, width), up (E, ff, width), down (E, width, ff), shared (T, width); returns (T, width).
+    The (token, choice) pairs are put in the order of their experts on the GPU (no number comes
+    back to the host), each expert's product runs over its rows in tiles, and a token's sum is
+    formed in float32 in the order of its choices, the shared addend last."""
+    _dev(h, chosen, weights, up, down, shared)
+    T, width = h.shape
+    E, ff = up.shape[0], up.shape[1]
+    top = chosen.shape[1]
+    _need(h.dtype in _DT and up.dtype == h.dtype and down.dtype == h.dtype and up.shape == (E, ff, width)
+          and down.shape == (E, width, ff), "up (E, ff, width) and down (E, width, ff) of h's dtype")
+    _need(chosen.shape == (T, top) and chosen.dtype == torch.int32 and weights.shape == (T, top)
+          and weights.dtype == torch.float32, "chosen int32 (T, top), weights float32 (T, top)")
+    _need(shared is None or (shared.shape == (T, width) and shared.dtype == h.dtype), "shared (T, width)")
+    _need(activation in GELU_KINDS, "activation erf or tanh")
+    out = torch.empty((T, width), dtype=h.dtype, device=h.device)
+    if not T:
+        return out
+    lib = library("moe")
+    P = T * top
+    max_tiles = -(-P // lib.q3_moe_tile_rows()) + E
+    book = torch.empty((E + 1 + 2 * P + 2 * max_tiles + 1,), dtype=torch.int32, device=h.device)
+    offsets, pair_of_slot, slot_of_pair = book[:E + 1], book[E + 1:E + 1 + P], book[E + 1 + P:E + 1 + 2 * P]
+    at = E + 1 + 2 * P
+    tile_expert, tile_first, n_tiles = book[at:at + max_tiles], book[at + max_tiles:at + 2 * max_tiles], book[at + 2 * max_tiles:]
+    stream = _stream()
+    _check(lib.q3_moe_align(_ptr(chosen), P, E, _ptr(offsets), _ptr(pair_of_slot), _ptr(slot_of_pair), _ptr(tile_expert),
+                            _ptr(tile_first), _ptr(n_tiles), stream), "moe_align")
+    hidden = torch.empty((P, ff), dtype=h.dtype, device=h.device)
+    _check(lib.q3_moe_linear(_ptr(h), _ptr(pair_of_slot), 1, top, _ptr(up), _ptr(hidden), _ptr(tile_expert),
+                             _ptr(tile_first), _ptr(offsets), _ptr(n_tiles), max_tiles, ff, width,
+                             GELU_KINDS[activation], _DT[h.dtype], stream), "moe_linear")
+    y = torch.empty((P, width), dtype=h.dtype, device=h.device)
+    _check(lib.q3_moe_linear(_ptr(hidden), _ptr(pair_of_slot), 0, 1, _ptr(down), _ptr(y), _ptr(tile_expert),
+                             _ptr(tile_first), _ptr(offsets), _ptr(n_tiles), max_tiles, width, ff, -1, _DT[h.dtype],
+                             stream), "moe_linear")
+    _check(lib.q3_moe_combine(_ptr(y), _ptr(slot_of_pair), _ptr(weights), _ptr(shared), _ptr(out), T, width, top,
+                              _DT[h.dtype], stream), "moe_combine")
     return out
 
 

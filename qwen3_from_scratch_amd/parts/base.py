@@ -105,6 +105,10 @@ class Part:
         stored dtype or converted to `dtype`; equal requests share one tensor."""
 
     def _name(self, leaf):
+        """The checkpoint name of the part's tensor `leaf`; with an empty leaf the prefix itself
+        (checkpoints that name a norm's or a table's only tensor by the part's own name)."""
+        if not leaf:
+            return self.prefix
         return self.prefix + "." + leaf if self.prefix else leaf
 
 
@@ -139,6 +143,21 @@ class UnscaledRows:
 
     def scale_args(self):
         return (self.sums, self.eps, self.width)
+
+
+@dataclass
+class StreamAddend:
+    """What the residual stream still lacks when a norm reads it next: `values` (T, width) in the
+    activation dtype, a part's result, which is first normalised by its root mean square with
+    `weight` and `eps` if `weight` is given (a block that also normalises what its parts return);
+    and `bias` (width,) float32, one vector for every row (what a model adds to the stream
+    between two layers). Either may be None. A norm that takes it as `delta` does the whole sum
+    in float32 in its own kernel, so the addend is never rounded on its way into the stream."""
+
+    values: torch.Tensor = None
+    weight: torch.Tensor = None
+    eps: float = 0.0
+    bias: torch.Tensor = None
 
 
 def build_part(spec, prefix, precision, device):

@@ -56,3 +56,43 @@ class PreNormBlock(Part):
         if sink is not None:
             return x, self.feed_forward.forward(h, batch, sink=sink)
         return x, self.feed_forward.forward(h, batch)
+
+
+@register_part("block", "sandwich")
+class SandwichBlock(Part):
+    """x = x + norm_1b(mixer(norm_1(x))); x = x + norm_2b(feed_forward(norm_2(x))): a norm before
+    and a norm behind each part. A layer without a feed-forward attaches the mixer and its two
+    norms only. What a part returns is not normalised by a kernel of its own: it travels as a
+    `StreamAddend` to the norm that reads the stream next (this block's second, or the next
+    block's first, or the model's last), which normalises it, adds it into the float32 stream and
+    normalises the stream in one pass; a norm that cannot take that (no `as_addend`) is applied
+    on the spot."""
+
+    graph_safe = True
+
+    def __init__(self, prefix, precision, device):
+        super().__init__(prefix, precision, device)
+        self.mixer = self.feed_forward = None
+        self.mixer_norm = self.mixer_out_norm = self.feed_forward_norm = self.feed_forward_out_norm = None
+
+    def attach(self, mixer, mixer_norm, mixer_out_norm, feed_forward=None, feed_forward_norm=None,
+               feed_forward_out_norm=None):
+        if (feed_forward is None) != (feed_forward_norm is None) or (feed_forward is None) != (feed_forward_out_norm is None):
+            raise ValueError("a feed-forward comes with a norm before and a norm behind it, or not at all")
+        self.mixer, self.mixer_norm, self.mixer_out_norm = mixer, mixer_norm, mixer_out_norm
+        self.feed_forward, self.feed_forward_norm = feed_forward, feed_forward_norm
+        self.feed_forward_out_norm = feed_forward_out_norm
+
+    @staticmethod
+    def _behind(norm, values):
+        if hasattr(norm, "as_addend"):
+            return norm.as_addend(values)
+        return norm.forward(values.float())
+
+    def forward(self, x, pending, batch, cache, next_norm=None):
+        mixed = self.mixer.forward(self.mixer_norm.forward(x, delta=pending), batch, cache)
+        pending = self._behind(self.mixer_out_norm, mixed)
+        if self.feed_forward is None:
+            return x, pending
+        fed = self.feed_forward.forward(self.feed_forward_norm.forward(x, delta=pending), batch)
+        return x, self._behind(self.feed_forward_out_norm, fed)

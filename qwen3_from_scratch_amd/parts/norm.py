@@ -4,7 +4,7 @@ import torch
 
 from .. import ops
 from ..config.registry import register_part
-from .base import NormSink, Part, TensorShape
+from .base import NormSink, Part, StreamAddend, TensorShape
 
 
 @register_part("norm", "rms")
@@ -17,23 +17,33 @@ class RMSNorm(Part):
 
     graph_safe = True
 
-    def __init__(self, prefix, precision, device, size, eps):
+    def __init__(self, prefix, precision, device, size, eps, leaf="weight"):
         super().__init__(prefix, precision, device)
         self.size = size
         self.eps = float(eps)
+        self.leaf = leaf            # the tensor's name below the prefix; "" if it is the prefix itself
         self.weight = None
 
     def tensors(self):
-        return {self._name("weight"): TensorShape((self.size,), "scale")}
+        return {self._name(self.leaf): TensorShape((self.size,), "scale")}
 
     def load(self, fetch):
-        self.weight = fetch(self._name("weight"))
+        self.weight = fetch(self._name(self.leaf))
 
     def forward(self, x, delta=None, rows=None):
         """Normalised rows in the activation dtype. With `delta`, x += delta
         first (in place, unless `rows` selects a subset: then x is left alone)."""
+        if isinstance(delta, StreamAddend):
+            return ops.rmsnorm_addend(x, self.weight, self.eps, self.precision.act, delta=delta.values,
+                                      delta_weight=delta.weight, delta_eps=delta.eps, bias=delta.bias, rows=rows,
+                                      write_back=rows is None)
         return ops.rmsnorm(x, self.weight, self.eps, self.precision.act, delta=delta,
                            rows=rows, write_back=rows is None)
+
+    def as_addend(self, values):
+        """`values` (a part's result) as what the stream still lacks, to be normalised by this norm
+        on its way in: the norm that reads the stream next does both in one kernel."""
+        return StreamAddend(values=values, weight=self.weight, eps=self.eps)
 
     def sink_for(self, x):
         """A NormSink for the residual `x` if this step may have the addition

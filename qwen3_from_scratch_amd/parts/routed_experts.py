@@ -1,0 +1,61 @@
+"""A feed-forward of many small experts, of which a router gives each token a few."""
+
+import torch
+
+from .. import ops
+from ..config.registry import register_part
+from .base import Part
+from .linear import LinearWeight
+
+
+@register_part("feed_forward", "routed_experts")
+class RoutedExperts(Part):
+    """z = W_router h (float32), s = softmax(z) over all experts; a token's `top` experts are
+    those with the largest scores, weighted by s / (their sum + 1e-20); each expert is
+    W_down act(W_up h) without biases; an optional shared expert of the same form (its own inner
+    size) serves every token and is added. `activation`: "erf" (the exact gelu) or "tanh".
+
+    Tensors: router (experts, hidden), e<i>.up (expert_ff, hidden), e<i>.down (hidden, expert_ff),
+    shared.up (shared_ff, hidden), shared.down (hidden, shared_ff). The experts' matrices are kept
+    stacked, (experts, ff, hidden) and (experts, hidden, ff); tokens are never counted on the
+    host, so a step is launches only.
+    """
+
+    graph_safe = True
+
+    def __init__(self, prefix, precision, device, hidden_size, experts, top, expert_ff, shared_ff=0, activation="erf"):
+        super().__init__(prefix, precision, device)
+        if not 1 <= top <= experts:
+            raise ValueError("top (%d) must lie in 1..experts (%d)" % (top, experts))
+        if activation not in ops.GELU_KINDS:
+            raise ValueError("activation is one of %s" % ", ".join(sorted(ops.GELU_KINDS)))
+        self.hidden_size, self.experts, self.top = hidden_size, experts, top
+        self.expert_ff, self.shared_ff, self.activation = expert_ff, shared_ff, activation
+        self.router = self.up = self.down = self.shared_up = self.shared_down = None
+
+    def tensors(self):
+        W = self.hidden_size
+        names = {self._name("router"): (self.experts, W)}
+        for e in range(self.experts):
+            names[self._name("e%d.up" % e)] = (self.expert_ff, W)
+            names[self._name("e%d.down" % e)] = (W, self.expert_ff)
+        if self.shared_ff:
+            names[self._name("shared.up")] = (self.shared_ff, W)
+            names[self._name("shared.down")] = (W, self.shared_ff)
+        return names
+
+    def load(self, fetch):
+        act, E = self.precision.act, self.experts
+        self.router = fetch(self._name("router"), act)
+        self.up = torch.stack([fetch(self._name("e%d.up" % e), act, keep=False) for e in range(E)]).contiguous()
+        self.down = torch.stack([fetch(self._name("e%d.down" % e), act, keep=False) for e in range(E)]).contiguous()
+        if self.shared_ff:
+            self.shared_up = LinearWeight(fetch(self._name("shared.up"), act), self.precision)
+            self.shared_down = LinearWeight(fetch(self._name("shared.down"), act), self.precision)
+
+    def forward(self, x, batch=None):
+        chosen, weights = ops.moe_route(x, self.router, self.top)
+        shared = None
+        if self.shared_ff:
+            shared = self.shared_down.forward(ops.gelu(self.shared_up.forward(x), self.activation))
+        return ops.moe_experts(x, chosen, weights, self.up, self.down, shared=shared, activation=self.activation)

@@ -176,5 +176,127 @@ def sample(logits, temperature, top_k, seed, counter, out=None, any_top_k=True):
     return res
 
 
+def rmsnorm_addend(x, weight, eps, out_dtype, delta=None, delta_weight=None, delta_eps=0.0, bias=None, rows=None,
+                   write_back=True, out=None):
+    src = x if rows is None else x[rows.long()]
+    if delta is not None:
+        d = (delta if rows is None else delta[rows.long()]).float()
+        if delta_weight is not None:
+            d = d * torch.rsqrt((d * d).mean(dim=-1, keepdim=True) + delta_eps) * delta_weight.float()
+        src = src + d
+    if bias is not None:
+        src = src + bias
+    if write_back and rows is None and (delta is not None or bias is not None):
+        x.copy_(src)
+    if weight is None:
+        return None
+    res = (src * torch.rsqrt((src * src).mean(dim=-1, keepdim=True) + eps) * weight.float()).to(out_dtype)
+    if out is not None:
+        out.copy_(res)
+        return out
+    return res
+
+
+GELU_KINDS = {"erf": 0, "tanh": 1}
+
+
+def gelu(x, kind="erf", out=None):
+    z = x.float()
+    if kind == "erf":
+        res = 0.5 * z * (1.0 + torch.erf(z / math.sqrt(2.0)))
+    else:
+        res = 0.5 * z * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * z ** 3)))
+    res = res.to(x.dtype)
+    if out is not None:
+        out.copy_(res)
+        return out
+    return res
+
+
+def _turn_pairs(t, positions, inv_freq, rot_factor):
+    """t (T, ..., n): pairs (2i, 2i + 1), i < len(inv_freq), turned by float32(position) * inv_freq[i]."""
+    n2 = 2 * inv_freq.shape[0]
+    angle = positions.float()[:, None] * inv_freq[None, :]
+    shape = (t.shape[0],) + (1,) * (t.dim() - 2) + (inv_freq.shape[0],)
+    cos, sin = (angle.cos() * rot_factor).view(shape), (angle.sin() * rot_factor).view(shape)
+    u, v = t[..., 0:n2:2], t[..., 1:n2:2]
+    turned = torch.stack((u * cos - v * sin, v * cos + u * sin), dim=-1).flatten(-2)
+    return torch.cat((turned, t[..., n2:]), dim=-1)
+
+
+def latent_prepare(down, q_rank, kv_rank, rot_dim, q_weight, kv_weight, eps, inv_freq, rot_factor, positions, seq_index,
+                   block_table=None, cache=None):
+    x = down.float()
+    a, b, tail = x[:, :q_rank], x[:, q_rank:q_rank + kv_rank], x[:, q_rank + kv_rank:]
+    cq = a * torch.rsqrt((a * a).mean(dim=-1, keepdim=True) + eps) * q_weight.float()
+    if cache is not None:
+        c = b * torch.rsqrt((b * b).mean(dim=-1, keepdim=True) + eps) * kv_weight.float()
+        row = torch.cat((c, _turn_pairs(tail, positions, inv_freq, rot_factor)), dim=-1)
+        page = cache.shape[1]
+        pos = positions.long()
+        pages = block_table[seq_index.long(), pos // page].long()
+        ok = pages >= 0
+        cache[pages[ok], (pos % page)[ok]] = row[ok].to(cache.dtype)
+    return cq.to(down.dtype)
+
+
+def headwise_linear(x, weight, out=None):
+    res = torch.einsum("thi,hio->tho", x.float(), weight.float()).to(x.dtype).contiguous()
+    if out is not None:
+        out.copy_(res)
+        return out
+    return res
+
+
+def rotate_heads(x, out, inv_freq, rot_factor, positions):
+    out.copy_(_turn_pairs(x.float(), positions, inv_freq, rot_factor).to(x.dtype))
+    return out
+
+
+def latent_attention(q, cache, value_dim, block_table, cu_seqlens_q, kv_lens, max_q_len, scale, window=0):
+    T, H, Dk = q.shape
+    page = cache.shape[1]
+    res = torch.zeros((T, H, value_dim), dtype=torch.float32, device=q.device)
+    cu, kvl = cu_seqlens_q.tolist(), kv_lens.tolist()
+    for b in range(len(kvl)):
+        q0, q1 = cu[b], cu[b + 1]
+        n, L = q1 - q0, kvl[b]
+        if n == 0:
+            continue
+        nblk = -(-L // page)
+        pages = block_table[b, :nblk].long().clamp(min=0)
+        rows = cache[pages].float().reshape(nblk * page, Dk)[:L]
+        qpos = torch.arange(L - n, L, device=q.device)[:, None]
+        kpos = torch.arange(L, device=q.device)[None, :]
+        hidden = kpos > qpos
+        if window > 0:
+            hidden = hidden | (qpos - kpos >= window)
+        s = torch.einsum("thd,sd->hts", q[q0:q1].float(), rows) * scale
+        p = torch.softmax(s.masked_fill(hidden[None], float("-inf")), dim=-1)
+        res[q0:q1] = torch.einsum("hts,sd->thd", p, rows[:, :value_dim])
+    return res.to(q.dtype)
+
+
+def moe_route(h, router, top):
+    s = torch.softmax(h.float() @ router.float().T, dim=-1)
+    best, chosen = torch.topk(s, top, dim=-1)
+    return chosen.to(torch.int32), best / (best.sum(dim=-1, keepdim=True) + 1e-20)
+
+
+def moe_experts(h, chosen, weights, up, down, shared=None, activation="erf"):
+    T, top = chosen.shape
+    out = torch.zeros((T, h.shape[1]), dtype=torch.float32, device=h.device)
+    for k in range(top):
+        e = chosen[:, k].long()
+        hidden = gelu(torch.einsum("ti,tfi->tf", h.float(), up[e].float()).to(h.dtype), activation)
+        y = torch.einsum("tf,twf->tw", hidden.float(), down[e].float()).to(h.dtype)
+        out += weights[:, k, None] * y.float()
+    if shared is not None:
+        out += shared.float()
+    return out.to(h.dtype)
+
+
 ALL = ("embed_rows", "swiglu", "rmsnorm", "rope_table", "qk_norm_rope_store",
-       "paged_attention", "decode_attention_takes", "linear", "linear_swiglu", "tile_weight", "sample")
+       "paged_attention", "decode_attention_takes", "linear", "linear_swiglu", "tile_weight", "sample",
+       "rmsnorm_addend", "gelu", "GELU_KINDS", "latent_prepare", "headwise_linear", "rotate_heads", "latent_attention",
+       "moe_route", "moe_experts")
