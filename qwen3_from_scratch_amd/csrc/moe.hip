@@ -185,6 +185,93 @@ __global__ __launch_bounds__(256) void moe_linear_kernel(const T* __restrict__ x
   }
 }
 
+// ---------------------------------------------------------------------------
+// The same products on the matrix cores (v_mfma_f32_16x16x32_bf16): bfloat16, K a multiple of 32.
+// out^T (columns x slots) = W_e (columns x K) . x^T (K x slots): 16 weight rows are the first
+// operand, 16 slots' rows of x the second, both straight from memory (a lane reads 16 bytes of
+// one row per step of 32 k). A tile has 32 slots (two second operands); a block's four wavefronts
+// each own NS slabs of 16 output columns, so every x operand serves NS matrix instructions and
+// every weight operand two. A lane ends up with four consecutive columns of one slot.
+// ---------------------------------------------------------------------------
+typedef __attribute__((ext_vector_type(8))) __bf16 moe_bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) float moe_f32x4_t;
+union MoePack {
+  uint4 u;
+  moe_bf16x8_t v;
+};
+#define MMA_TM 32
+
+template <int NS>
+__global__ __launch_bounds__(256) void moe_linear_mma_kernel(
+    const bf16_t* __restrict__ x, const int* __restrict__ pair_of_slot, int gather, int pairs_per_row,
+    const bf16_t* __restrict__ w, bf16_t* __restrict__ out, const int* __restrict__ tile_expert,
+    const int* __restrict__ tile_first, const int* __restrict__ offsets, const int* __restrict__ n_tiles, int N, int K,
+    int act) {
+  const int tile = blockIdx.x;
+  if (tile >= n_tiles[0]) return;
+  const int e = tile_expert[tile];
+  const int first = tile_first[tile];
+  const int rows = min(MMA_TM, offsets[e + 1] - first);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int col = lane & 15, grp = lane >> 4;
+  const bf16_t* xr[2];
+#pragma unroll
+  for (int mt = 0; mt < 2; ++mt) {
+    const int m = 16 * mt + col;
+    xr[mt] = nullptr;
+    if (m < rows) {
+      const int src = gather ? pair_of_slot[first + m] / pairs_per_row : first + m;
+      xr[mt] = x + (size_t)src * K + 8 * grp;
+    }
+  }
+  const int n_base = (blockIdx.y * 4 + wave) * (16 * NS);
+  if (n_base >= N) return;
+  const bf16_t* wr[NS];
+#pragma unroll
+  for (int ns = 0; ns < NS; ++ns) {
+    const int n = n_base + 16 * ns + col;
+    wr[ns] = n < N ? w + ((size_t)e * N + n) * K + 8 * grp : nullptr;
+  }
+  moe_f32x4_t acc[2][NS];
+#pragma unroll
+  for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+    for (int ns = 0; ns < NS; ++ns) acc[mt][ns] = moe_f32x4_t{0.f, 0.f, 0.f, 0.f};
+  const bool two = rows > 16;
+#pragma unroll 4
+  for (int k0 = 0; k0 < K; k0 += 32) {
+    MoePack a[NS], b[2];
+#pragma unroll
+    for (int ns = 0; ns < NS; ++ns)
+      a[ns].u = wr[ns] ? *reinterpret_cast<const uint4*>(wr[ns] + k0) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt)
+      b[mt].u = xr[mt] ? *reinterpret_cast<const uint4*>(xr[mt] + k0) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+    for (int ns = 0; ns < NS; ++ns) {
+      acc[0][ns] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[ns].v, b[0].v, acc[0][ns], 0, 0, 0);
+      if (two) acc[1][ns] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[ns].v, b[1].v, acc[1][ns], 0, 0, 0);
+    }
+  }
+#pragma unroll
+  for (int mt = 0; mt < 2; ++mt) {
+    const int m = 16 * mt + col;
+    if (m >= rows) continue;
+#pragma unroll
+    for (int ns = 0; ns < NS; ++ns) {
+      const int n = n_base + 16 * ns + 4 * grp;
+      bf16_t* o = out + (size_t)(first + m) * N + n;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (n + i < N) {
+          const float v = acc[mt][ns][i];
+          o[i] = float_to_bf16(act >= 0 ? moe_gelu(v, act) : v);
+        }
+      }
+    }
+  }
+}
+
 // out[t, :] = sum_k weights[t, k] * y[slot_of_pair[t * top + k], :] (+ shared[t, :]), float32 sums in
 // the order k = 0, 1, ..., the shared expert last; rounded once.
 template <typename T>
@@ -215,13 +302,34 @@ extern "C" int q3_moe_route(const void* h, const void* router, int n_tokens, int
   return q3_launch_status();
 }
 
-extern "C" int q3_moe_tile_rows() { return MOE_BM; }
+// Slots per tile: 16 for the float32 multiply-add kernel, 32 for the matrix-core kernel.
+extern "C" int q3_moe_tile_rows(int matrix_cores) { return matrix_cores ? MMA_TM : MOE_BM; }
 
-extern "C" int q3_moe_align(const int* chosen, int P, int E, int* offsets, int* pair_of_slot, int* slot_of_pair,
-                            int* tile_expert, int* tile_first, int* n_tiles, hipStream_t stream) {
-  if (P <= 0 || E <= 0 || E > 4096) return Q3_ERR_BAD_ARGUMENT;
-  hipLaunchKernelGGL(moe_align_kernel, dim3(1), dim3(1024), (size_t)2 * E * sizeof(int), stream, chosen, P, E, MOE_BM,
-                     offsets, pair_of_slot, slot_of_pair, tile_expert, tile_first, n_tiles);
+extern "C" int q3_moe_align(const int* chosen, int P, int E, int tile_rows, int* offsets, int* pair_of_slot,
+                            int* slot_of_pair, int* tile_expert, int* tile_first, int* n_tiles, hipStream_t stream) {
+  if (P <= 0 || E <= 0 || E > 4096 || (tile_rows != MOE_BM && tile_rows != MMA_TM)) return Q3_ERR_BAD_ARGUMENT;
+  hipLaunchKernelGGL(moe_align_kernel, dim3(1), dim3(1024), (size_t)2 * E * sizeof(int), stream, chosen, P, E,
+                     tile_rows, offsets, pair_of_slot, slot_of_pair, tile_expert, tile_first, n_tiles);
+  return q3_launch_status();
+}
+
+// The matrix-core product: bfloat16, K a multiple of 32, tiles of 32 slots.
+extern "C" int q3_moe_linear_mma(const void* x, const int* pair_of_slot, int gather, int pairs_per_row, const void* w,
+                                 void* out, const int* tile_expert, const int* tile_first, const int* offsets,
+                                 const int* n_tiles, int max_tiles, int N, int K, int act, hipStream_t stream) {
+  if (max_tiles <= 0 || N <= 0 || K <= 0 || K % 32 || pairs_per_row <= 0 || act < -1 || act > 1)
+    return Q3_ERR_BAD_ARGUMENT;
+  // few blocks (steps of few tokens): one slab of 16 columns per wavefront, so that more blocks stream the weights
+  const bool narrow = (long)max_tiles * ((N + 127) / 128) < 512;
+  const int per_block = narrow ? 64 : 128;
+  const dim3 grid(max_tiles, (N + per_block - 1) / per_block);
+  if (grid.y > 65535) return Q3_ERR_UNSUPPORTED;
+  if (narrow)
+    hipLaunchKernelGGL(moe_linear_mma_kernel<1>, grid, dim3(256), 0, stream, (const bf16_t*)x, pair_of_slot, gather,
+                       pairs_per_row, (const bf16_t*)w, (bf16_t*)out, tile_expert, tile_first, offsets, n_tiles, N, K, act);
+  else
+    hipLaunchKernelGGL(moe_linear_mma_kernel<2>, grid, dim3(256), 0, stream, (const bf16_t*)x, pair_of_slot, gather,
+                       pairs_per_row, (const bf16_t*)w, (bf16_t*)out, tile_expert, tile_first, offsets, n_tiles, N, K, act);
   return q3_launch_status();
 }
 

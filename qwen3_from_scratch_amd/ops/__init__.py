@@ -500,22 +500,31 @@ def moe_experts(h, chosen, weights, up, down, shared=None, activation="erf"):
         return out
     lib = library("moe")
     P = T * top
-    max_tiles = -(-P // lib.q3_moe_tile_rows()) + E
+    # bfloat16 with inner sizes in steps of 32: the matrix-core kernel over tiles of 32 slots;
+    # anything else: float32 multiply-adds over tiles of 16
+    cores = h.dtype == torch.bfloat16 and width % 32 == 0 and ff % 32 == 0
+    tile_rows = lib.q3_moe_tile_rows(1 if cores else 0)
+    max_tiles = -(-P // tile_rows) + E
     book = torch.empty((E + 1 + 2 * P + 2 * max_tiles + 1,), dtype=torch.int32, device=h.device)
     offsets, pair_of_slot, slot_of_pair = book[:E + 1], book[E + 1:E + 1 + P], book[E + 1 + P:E + 1 + 2 * P]
     at = E + 1 + 2 * P
     tile_expert, tile_first, n_tiles = book[at:at + max_tiles], book[at + max_tiles:at + 2 * max_tiles], book[at + 2 * max_tiles:]
     stream = _stream()
-    _check(lib.q3_moe_align(_ptr(chosen), P, E, _ptr(offsets), _ptr(pair_of_slot), _ptr(slot_of_pair), _ptr(tile_expert),
-                            _ptr(tile_first), _ptr(n_tiles), stream), "moe_align")
+    _check(lib.q3_moe_align(_ptr(chosen), P, E, tile_rows, _ptr(offsets), _ptr(pair_of_slot), _ptr(slot_of_pair),
+                            _ptr(tile_expert), _ptr(tile_first), _ptr(n_tiles), stream), "moe_align")
     hidden = torch.empty((P, ff), dtype=h.dtype, device=h.device)
-    _check(lib.q3_moe_linear(_ptr(h), _ptr(pair_of_slot), 1, top, _ptr(up), _ptr(hidden), _ptr(tile_expert),
-                             _ptr(tile_first), _ptr(offsets), _ptr(n_tiles), max_tiles, ff, width,
-                             GELU_KINDS[activation], _DT[h.dtype], stream), "moe_linear")
     y = torch.empty((P, width), dtype=h.dtype, device=h.device)
-    _check(lib.q3_moe_linear(_ptr(hidden), _ptr(pair_of_slot), 0, 1, _ptr(down), _ptr(y), _ptr(tile_expert),
-                             _ptr(tile_first), _ptr(offsets), _ptr(n_tiles), max_tiles, width, ff, -1, _DT[h.dtype],
-                             stream), "moe_linear")
+    tiles = (_ptr(tile_expert), _ptr(tile_first), _ptr(offsets), _ptr(n_tiles), max_tiles)
+    if cores:
+        _check(lib.q3_moe_linear_mma(_ptr(h), _ptr(pair_of_slot), 1, top, _ptr(up), _ptr(hidden), *tiles, ff, width,
+                                     GELU_KINDS[activation], stream), "moe_linear")
+        _check(lib.q3_moe_linear_mma(_ptr(hidden), _ptr(pair_of_slot), 0, 1, _ptr(down), _ptr(y), *tiles, width, ff,
+                                     -1, stream), "moe_linear")
+    else:
+        _check(lib.q3_moe_linear(_ptr(h), _ptr(pair_of_slot), 1, top, _ptr(up), _ptr(hidden), *tiles, ff, width,
+                                 GELU_KINDS[activation], _DT[h.dtype], stream), "moe_linear")
+        _check(lib.q3_moe_linear(_ptr(hidden), _ptr(pair_of_slot), 0, 1, _ptr(down), _ptr(y), *tiles, width, ff, -1,
+                                 _DT[h.dtype], stream), "moe_linear")
     _check(lib.q3_moe_combine(_ptr(y), _ptr(slot_of_pair), _ptr(weights), _ptr(shared), _ptr(out), T, width, top,
                               _DT[h.dtype], stream), "moe_combine")
     return out
