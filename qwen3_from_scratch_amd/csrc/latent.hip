@@ -66,10 +66,11 @@ __global__ void latent_prepare_kernel(const T* __restrict__ down, int q_rank, in
 }
 
 // ---------------------------------------------------------------------------
-// y[t, h, :] = W[h]^T x[t, h, :] for every head: x rows of `I` numbers at x + t * x_row + h * x_head,
-// W (H, I, O) row-major (the summed index first), y rows of `O` numbers at out + t * out_row +
-// h * out_head. One block: 16 tokens of one head, up to 256 output columns; the tokens' inputs
-// wait in shared memory, each thread owns one output column and walks I in order.
+// y[t, h, :] = W[h] x[t, h, :] for every head: x rows of `I` numbers at x + t * x_row + h * x_head,
+// W (H, O, I) row-major (a result's weights side by side), y rows of `O` numbers at
+// out + t * out_row + h * out_head. The general kernel: one block is 16 tokens of one head and up
+// to 256 output columns; the tokens' inputs wait in shared memory, each thread owns one output
+// column and walks I in order with float32 sums.
 // ---------------------------------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(256) void headwise_linear_kernel(const T* __restrict__ x, long x_row, int x_head,
@@ -89,14 +90,85 @@ __global__ __launch_bounds__(256) void headwise_linear_kernel(const T* __restric
   float acc[16];
 #pragma unroll
   for (int m = 0; m < 16; ++m) acc[m] = 0.f;
-  const T* wh = w + (size_t)h * I * O + o;
+  const T* wh = w + ((size_t)h * O + o) * I;
   for (int i = 0; i < I; ++i) {
-    const float wv = to_float(wh[(size_t)i * O]);
+    const float wv = to_float(wh[i]);
 #pragma unroll
     for (int m = 0; m < 16; ++m) acc[m] += xs[m * I + i] * wv;
   }
   for (int m = 0; m < rows; ++m)
     out[(size_t)(m0 + m) * out_row + (size_t)h * out_head + o] = from_float<T>(acc[m]);
+}
+
+// The same on the matrix cores (v_mfma_f32_16x16x32_bf16): bfloat16, I a multiple of 32, rows of x
+// that start at multiples of 16 bytes. y^T (columns x tokens) = W_h (columns x I) . x_h^T: 16 weight
+// rows are the first operand, 16 tokens' rows the second, both straight from memory. A wavefront
+// owns 16 MT tokens and 128 output columns of one head (8 slabs of 16): per step of 32 k it reads
+// MT operands of x and 8 of W for 8 MT matrix instructions.
+typedef __attribute__((ext_vector_type(8))) __bf16 lat_bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) float lat_f32x4_t;
+union LatPack {
+  uint4 u;
+  uint2 h[2];
+  lat_bf16x8_t v;
+  __bf16 e[8];
+};
+
+template <int MT>
+__global__ __launch_bounds__(256) void headwise_linear_mma_kernel(const bf16_t* __restrict__ x, long x_row, int x_head,
+                                                                  const bf16_t* __restrict__ w,
+                                                                  bf16_t* __restrict__ out, long out_row, int out_head,
+                                                                  int n_rows, int I, int O) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int col = lane & 15, grp = lane >> 4;
+  const int h = blockIdx.y;
+  const int t0 = (blockIdx.x * 4 + wave) * 16 * MT;
+  if (t0 >= n_rows) return;
+  const int o_base = blockIdx.z * 128;
+  const bf16_t* xr[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int t = t0 + 16 * mt + col;
+    xr[mt] = t < n_rows ? x + (size_t)t * x_row + (size_t)h * x_head + 8 * grp : nullptr;
+  }
+  const bf16_t* wr[8];
+#pragma unroll
+  for (int s = 0; s < 8; ++s) {
+    const int o = o_base + 16 * s + col;
+    wr[s] = o < O ? w + ((size_t)h * O + o) * I + 8 * grp : nullptr;
+  }
+  lat_f32x4_t acc[MT][8];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int s = 0; s < 8; ++s) acc[mt][s] = lat_f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 2
+  for (int k0 = 0; k0 < I; k0 += 32) {
+    LatPack a[8], b[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+      b[mt].u = xr[mt] ? *reinterpret_cast<const uint4*>(xr[mt] + k0) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+    for (int s = 0; s < 8; ++s) a[s].u = wr[s] ? *reinterpret_cast<const uint4*>(wr[s] + k0) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+    for (int s = 0; s < 8; ++s)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+        acc[mt][s] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[s].v, b[mt].v, acc[mt][s], 0, 0, 0);
+  }
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int t = t0 + 16 * mt + col;
+    if (t >= n_rows) continue;
+    bf16_t* o_row = out + (size_t)t * out_row + (size_t)h * out_head;
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      const int o = o_base + 16 * s + 4 * grp;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (o + i < O) o_row[o + i] = float_to_bf16(acc[mt][s][i]);
+    }
+  }
 }
 
 // The rotated tail of every query head: out[t, h, j] = rotate(x[t, h, j]) for the `rot_dim`
@@ -248,6 +320,175 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(const T* __restrict__ 
   }
 }
 
+// ---------------------------------------------------------------------------
+// The matrix-core kernel (v_mfma_f32_16x16x32_bf16): bfloat16, Dk a multiple of 32, Dv of 16.
+// A block of four wavefronts serves 64 consecutive (token, head) rows of one sequence, 16 per
+// wavefront, against tiles of 32 cached rows that start at absolute positions in steps of 32.
+// Every tile goes from the cache to shared memory once for all 64 rows and twice over: as it is
+// (keys: a lane's operand is 16 bytes of one cached row) and transposed (values: a lane's
+// operand is two runs of four keys of one column), because the first product sums over a row's
+// numbers and the second over the keys:
+//   S^T (keys x rows)  = K (keys x Dk) . Q^T          first operand K rows, second Q rows (registers)
+//   O^T (Dv x rows)   += V^T (Dv x keys) . P^T        first operand V^T rows, second P
+// Both leave a query row in the lanes l, l + 16, l + 32, l + 48, so a row's statistics, weights and
+// sums stay where they are. After S^T a lane holds the scores of keys 4g..4g+3 of both 16-key
+// halves (g = lane / 16); the second product numbers its summed index so that these are the
+// lane's eight, and reads V^T accordingly. Scores, maxima, sums and the output sums are float32;
+// weights are rounded to bfloat16 as the second product's operand.
+// ---------------------------------------------------------------------------
+#define LMA_ROWS 64
+#define LMA_BN 32
+#define LMA_KPAD 8
+#define LMA_VLD 40   // halfwords per transposed row: 32 keys and 8 of padding
+
+template <int KS, int NV>
+__global__ __launch_bounds__(256) void latent_attn_mma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
+                                                              const bf16_t* __restrict__ cache, int num_pages,
+                                                              const int* __restrict__ block_table, int bt_stride,
+                                                              const int* __restrict__ cu_q,
+                                                              const int* __restrict__ kv_lens, int H, int Dk, int Dv,
+                                                              int page, float scale_log2, int window) {
+  extern __shared__ __align__(16) unsigned char lma_smem[];
+  const int b = blockIdx.y;
+  const int q0 = cu_q[b];
+  const int q_len = cu_q[b + 1] - q0;
+  const int n_rows = q_len * H;
+  const int m0 = blockIdx.x * LMA_ROWS;
+  if (m0 >= n_rows) return;
+  const int kv_len = kv_lens[b];
+  const int base_pos = kv_len - q_len;
+  const int ldk = Dk + LMA_KPAD;                              // halfwords per key row
+  bf16_t* kt = reinterpret_cast<bf16_t*>(lma_smem);           // [32][ldk]
+  bf16_t* vt = kt + LMA_BN * ldk;                             // [Dv][LMA_VLD]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int col = lane & 15, grp = lane >> 4;
+  const int ks = Dk >> 5, nv = Dv >> 4;
+
+  // the block's span of keys, and this wavefront's
+  const int block_last = min(m0 + LMA_ROWS, n_rows) - 1;
+  const int k_end = base_pos + block_last / H + 1;
+  int k_begin = window > 0 ? max(0, base_pos + m0 / H - window + 1) : 0;
+  k_begin -= k_begin % LMA_BN;
+  const int w0 = m0 + 16 * wave;
+  const bool wave_active = w0 < n_rows;
+  const int wave_last = min(w0 + 16, n_rows) - 1;
+  const int wave_k_end = wave_active ? base_pos + wave_last / H + 1 : 0;
+  const int wave_k_begin = (wave_active && window > 0) ? max(0, base_pos + w0 / H - window + 1) : 0;
+
+  const int R = w0 + col;
+  const bool valid = R < n_rows;
+  const int Rc = valid ? R : (wave_active ? wave_last : 0);
+  const int tok = Rc / H, head = Rc - tok * H;
+  const int pos = base_pos + tok;
+  LatPack qreg[KS];
+  {
+    const bf16_t* qr = q + ((size_t)(q0 + tok) * H + head) * Dk + 8 * grp;
+#pragma unroll
+    for (int i = 0; i < KS; ++i)
+      qreg[i].u = (i < ks && wave_active) ? *reinterpret_cast<const uint4*>(qr + 32 * i) : make_uint4(0, 0, 0, 0);
+  }
+  lat_f32x4_t acc[NV];
+#pragma unroll
+  for (int nb = 0; nb < NV; ++nb) acc[nb] = lat_f32x4_t{0.f, 0.f, 0.f, 0.f};
+  float m_run = -INFINITY, l_run = 0.f;
+  const int chunks_per_key = Dk >> 3;
+  const int chunks = LMA_BN * chunks_per_key;
+
+  for (int kt0 = k_begin; kt0 < k_end; kt0 += LMA_BN) {
+    __syncthreads();
+    for (int c = threadIdx.x; c < chunks; c += 256) {
+      const int j = c / chunks_per_key, d0 = (c - j * chunks_per_key) * 8;
+      const int kj = kt0 + j;
+      LatPack v;
+      v.u = make_uint4(0, 0, 0, 0);
+      if (kj < k_end) {
+        const int pg = block_table[(size_t)b * bt_stride + kj / page];
+        if (pg >= 0 && pg < num_pages)
+          v.u = *reinterpret_cast<const uint4*>(cache + ((size_t)pg * page + kj % page) * Dk + d0);
+      }
+      *reinterpret_cast<uint4*>(kt + j * ldk + d0) = v.u;
+      if (d0 < Dv) {
+        const unsigned short* e = reinterpret_cast<const unsigned short*>(&v.u);
+        unsigned short* dst = reinterpret_cast<unsigned short*>(vt) + d0 * LMA_VLD + j;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) dst[i * LMA_VLD] = e[i];
+      }
+    }
+    __syncthreads();
+    if (!wave_active || kt0 >= wave_k_end || kt0 + LMA_BN <= wave_k_begin) continue;
+    lat_f32x4_t sc[2];
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+      lat_f32x4_t c = lat_f32x4_t{0.f, 0.f, 0.f, 0.f};
+      const bf16_t* kr = kt + (16 * kb + col) * ldk + 8 * grp;
+#pragma unroll
+      for (int i = 0; i < KS; ++i) {
+        if (i < ks) {
+          LatPack a;
+          a.u = *reinterpret_cast<const uint4*>(kr + 32 * i);
+          c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, qreg[i].v, c, 0, 0, 0);
+        }
+      }
+      sc[kb] = c;
+    }
+    float v[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int key = kt0 + 16 * (j >> 2) + 4 * grp + (j & 3);
+      bool seen = valid && key <= pos;
+      if (window > 0 && pos - key >= window) seen = false;
+      v[j] = seen ? sc[j >> 2][j & 3] : -INFINITY;
+    }
+    float mx = fmaxf(fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3])), fmaxf(fmaxf(v[4], v[5]), fmaxf(v[6], v[7])));
+    mx = quad_rows_max(mx);
+    const float m_new = fmaxf(m_run, mx * scale_log2);
+    LatPack p;
+    float sum = 0.f;
+    float alpha = 1.f;
+    if (m_new > -INFINITY) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float e = exp2f(fmaf(v[j], scale_log2, -m_new));
+        sum += e;
+        p.e[j] = (__bf16)e;
+      }
+      alpha = exp2f(m_run - m_new);
+    } else {
+      p.u = make_uint4(0, 0, 0, 0);
+    }
+    sum = quad_rows_sum(sum);
+    l_run = l_run * alpha + sum;
+    m_run = m_new;
+#pragma unroll
+    for (int nb = 0; nb < NV; ++nb) {
+      if (nb < nv) {
+        acc[nb] *= alpha;
+        const bf16_t* vr = vt + (16 * nb + col) * LMA_VLD + 4 * grp;
+        LatPack a;
+        a.h[0] = *reinterpret_cast<const uint2*>(vr);
+        a.h[1] = *reinterpret_cast<const uint2*>(vr + 16);
+        acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, p.v, acc[nb], 0, 0, 0);
+      }
+    }
+  }
+  if (valid) {
+    const float inv = 1.f / l_run;
+    bf16_t* o = out + ((size_t)(q0 + tok) * H + head) * Dv + 4 * grp;
+#pragma unroll
+    for (int nb = 0; nb < NV; ++nb) {
+      if (nb < nv) {
+        union {
+          uint2 u;
+          bf16_t e[4];
+        } pk;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) pk.e[i] = float_to_bf16(acc[nb][i] * inv);
+        *reinterpret_cast<uint2*>(o + 16 * nb) = pk.u;
+      }
+    }
+  }
+}
+
 static int raise_shared_memory(const void* kernel, size_t smem) {
   if (smem <= 48 * 1024) return 0;
   if (smem > 160 * 1024) return Q3_ERR_UNSUPPORTED;
@@ -279,8 +520,23 @@ extern "C" int q3_latent_prepare(const void* down, int T, int q_rank, int kv_ran
 }
 
 extern "C" int q3_headwise_linear(const void* x, long x_row, int x_head, const void* w, void* out, long out_row,
-                                  int out_head, int n_rows, int H, int I, int O, int dtype, hipStream_t stream) {
+                                  int out_head, int n_rows, int H, int I, int O, int dtype, int matrix_cores,
+                                  hipStream_t stream) {
   if (n_rows <= 0 || H <= 0 || I <= 0 || O <= 0 || H > 65535) return Q3_ERR_BAD_ARGUMENT;
+  if (matrix_cores) {
+    // the caller has checked: bfloat16, I in steps of 32, rows of x at multiples of 16 bytes
+    if (dtype != Q3_BF16 || I % 32 || x_row % 8 || x_head % 8 || ((uintptr_t)x & 15) || ((uintptr_t)w & 15))
+      return Q3_ERR_BAD_ARGUMENT;
+    const int zs = (O + 127) / 128;
+    if (n_rows > 64) {
+      hipLaunchKernelGGL(headwise_linear_mma_kernel<2>, dim3((n_rows + 127) / 128, H, zs), dim3(256), 0, stream,
+                         (const bf16_t*)x, x_row, x_head, (const bf16_t*)w, (bf16_t*)out, out_row, out_head, n_rows, I, O);
+    } else {
+      hipLaunchKernelGGL(headwise_linear_mma_kernel<1>, dim3((n_rows + 63) / 64, H, zs), dim3(256), 0, stream,
+                         (const bf16_t*)x, x_row, x_head, (const bf16_t*)w, (bf16_t*)out, out_row, out_head, n_rows, I, O);
+    }
+    return q3_launch_status();
+  }
   const size_t smem = (size_t)16 * I * sizeof(float);
   int threads = 64;
   while (threads < 256 && threads < O) threads *= 2;
@@ -323,12 +579,43 @@ static int launch_latent_attn(const void* q, void* out, const void* cache, int n
   return q3_launch_status();
 }
 
+template <int KS, int NV>
+static int launch_latent_attn_mma(const void* q, void* out, const void* cache, int num_pages, const int* block_table,
+                                  int bt_stride, const int* cu_q, const int* kv_lens, int B, int H, int Dk, int Dv,
+                                  int page, float scale, int window, int max_q_len, hipStream_t stream) {
+  const size_t smem = (size_t)(LMA_BN * (Dk + LMA_KPAD) + Dv * LMA_VLD) * sizeof(bf16_t);
+  int e = raise_shared_memory((const void*)latent_attn_mma_kernel<KS, NV>, smem);
+  if (e) return e;
+  const long tiles = ((long)max_q_len * H + LMA_ROWS - 1) / LMA_ROWS;
+  if (tiles > 0x7fffffffL || B > 65535) return Q3_ERR_UNSUPPORTED;
+  hipLaunchKernelGGL((latent_attn_mma_kernel<KS, NV>), dim3((unsigned)tiles, B), dim3(256), smem, stream,
+                     (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)cache, num_pages, block_table, bt_stride, cu_q,
+                     kv_lens, H, Dk, Dv, page, scale * 1.44269504088896341f, window);
+  return q3_launch_status();
+}
+
+// Whether the matrix-core kernel serves these sizes.
+extern "C" int q3_latent_attention_fast_path(int Dk, int Dv, int dtype) {
+  return dtype == Q3_BF16 && Dk % 32 == 0 && Dv % 16 == 0 && Dv <= Dk && Dk <= 576 && Dv <= 512;
+}
+
 extern "C" int q3_latent_attention(const void* q, void* out, const void* cache, int num_pages, const int* block_table,
                                    int bt_stride, const int* cu_q, const int* kv_lens, int B, int H, int Dk, int Dv,
-                                   int page, float scale, int window, int max_q_len, int dtype, hipStream_t stream) {
+                                   int page, float scale, int window, int max_q_len, int dtype, int general,
+                                   hipStream_t stream) {
   if (B <= 0 || H <= 0 || Dk <= 0 || Dv <= 0 || Dv > Dk || page <= 0 || max_q_len <= 0 || window < 0)
     return Q3_ERR_BAD_ARGUMENT;
   if (Dv > 1024) return Q3_ERR_UNSUPPORTED;
+  if (!general && q3_latent_attention_fast_path(Dk, Dv, dtype)) {
+    if (Dk <= 192 && Dv <= 128)
+      return launch_latent_attn_mma<6, 8>(q, out, cache, num_pages, block_table, bt_stride, cu_q, kv_lens, B, H, Dk, Dv,
+                                          page, scale, window, max_q_len, stream);
+    if (Dk <= 320 && Dv <= 256)
+      return launch_latent_attn_mma<10, 16>(q, out, cache, num_pages, block_table, bt_stride, cu_q, kv_lens, B, H, Dk,
+                                            Dv, page, scale, window, max_q_len, stream);
+    return launch_latent_attn_mma<18, 32>(q, out, cache, num_pages, block_table, bt_stride, cu_q, kv_lens, B, H, Dk, Dv,
+                                          page, scale, window, max_q_len, stream);
+  }
   Q3_DISPATCH_DTYPE(dtype, TT, {
     if (Dv <= 128)
       return launch_latent_attn<TT, 8>(q, out, cache, num_pages, block_table, bt_stride, cu_q, kv_lens, B, H, Dk, Dv,

@@ -397,22 +397,25 @@ def latent_prepare(down, q_rank, kv_rank, rot_dim, q_weight, kv_weight, eps, inv
 
 
 def headwise_linear(x, weight, out=None):
-    """out[t, h, :] = weight[h]^T x[t, h, :]: x (T, H, I) seen through strides (its last axis
-    contiguous), weight (H, I, O) contiguous, out (T, H, O) likewise seen through strides; float32
-    sums in the order of I."""
+    """out[t, h, :] = weight[h] x[t, h, :]: x (T, H, I) seen through strides (its last axis
+    contiguous), weight (H, O, I) contiguous, out (T, H, O) likewise seen through strides; float32
+    sums. bfloat16 with I in steps of 32 and rows of x that start at multiples of 16 bytes runs on
+    the matrix cores, everything else as float32 multiply-adds in the order of I."""
     _dev(weight)
     _need(x.is_cuda and x.dim() == 3 and x.stride(2) == 1 and weight.dim() == 3 and x.dtype in _DT
-          and weight.dtype == x.dtype, "x (T, H, I) with a contiguous last axis, weight (H, I, O), one dtype")
+          and weight.dtype == x.dtype, "x (T, H, I) with a contiguous last axis, weight (H, O, I), one dtype")
     T, H, I = x.shape
-    O = weight.shape[2]
-    _need(weight.shape == (H, I, O), "weight must be (H, I, O)")
+    O = weight.shape[1]
+    _need(weight.shape == (H, O, I), "weight must be (H, O, I)")
     if out is None:
         out = torch.empty((T, H, O), dtype=x.dtype, device=x.device)
     _need(out.is_cuda and out.shape == (T, H, O) and out.stride(2) == 1 and out.dtype == x.dtype, "out must be (T, H, O)")
+    cores = (x.dtype == torch.bfloat16 and I % 32 == 0 and x.stride(0) % 8 == 0 and x.stride(1) % 8 == 0
+             and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0)
     if T:
         _check(library("latent").q3_headwise_linear(
             _ptr(x), ctypes.c_long(x.stride(0)), x.stride(1), _ptr(weight), _ptr(out), ctypes.c_long(out.stride(0)),
-            out.stride(1), T, H, I, O, _DT[x.dtype], _stream()), "headwise_linear")
+            out.stride(1), T, H, I, O, _DT[x.dtype], 1 if cores else 0, _stream()), "headwise_linear")
     return out
 
 
@@ -434,14 +437,17 @@ def rotate_heads(x, out, inv_freq, rot_factor, positions):
     return out
 
 
-def latent_attention(q, cache, value_dim, block_table, cu_seqlens_q, kv_lens, max_q_len, scale, window=0):
+def latent_attention(q, cache, value_dim, block_table, cu_seqlens_q, kv_lens, max_q_len, scale, window=0,
+                     general=False):
     """Causal softmax attention of every head's query rows over one shared sequence of cached rows.
 
     q (T, H, Dk) contiguous; cache (pages, page, Dk): the row of sequence b's position j lies in
     page block_table[b, j // page]; a row is the key in full and the value in its first
     `value_dim` numbers. The query of token i of sequence b (position kv_lens[b] - q_len + i) sees
     positions j <= its own and, with window > 0, only those fewer than `window` behind it.
-    Returns (T, H, value_dim). Float32 scores, statistics and sums."""
+    Returns (T, H, value_dim). Float32 scores, statistics and sums. bfloat16 with Dk in steps of 32
+    (up to 576) and value_dim in steps of 16 (up to 512) runs on the matrix cores; everything
+    else, and everything with `general=True`, takes the kernel of float32 multiply-adds."""
     _dev(q, cache, block_table, cu_seqlens_q, kv_lens)
     _need(q.dim() == 3 and q.dtype in _DT and cache.dim() == 3 and cache.dtype == q.dtype
           and cache.shape[2] == q.shape[2], "q (T, H, Dk) and cache (pages, page, Dk) of one dtype")
@@ -457,7 +463,7 @@ def latent_attention(q, cache, value_dim, block_table, cu_seqlens_q, kv_lens, ma
         _check(library("latent").q3_latent_attention(
             _ptr(q), _ptr(out), _ptr(cache), cache.shape[0], _ptr(block_table), block_table.shape[1],
             _ptr(cu_seqlens_q), _ptr(kv_lens), B, H, Dk, value_dim, cache.shape[1], ctypes.c_float(scale), int(window),
-            int(max_q_len), _DT[q.dtype], _stream()), "latent_attention")
+            int(max_q_len), _DT[q.dtype], 1 if general else 0, _stream()), "latent_attention")
     return out
 
 

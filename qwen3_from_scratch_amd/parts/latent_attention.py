@@ -70,9 +70,9 @@ class LatentAttention(Part):
         down = torch.cat((fetch(self._name("dq"), act, keep=False), fetch(self._name("dkv"), act, keep=False)), dim=0)
         self.down = LinearWeight(down.contiguous(), self.precision)
         self.uq = LinearWeight(fetch(self._name("uq"), act), self.precision)
-        # per head (summed index, result index): uk as stored, uv transposed
-        self.uk = fetch(self._name("uk"), act).view(H, self.dim, self.kv_rank).contiguous()
-        self.uv = fetch(self._name("uv"), act, keep=False).view(H, self.vdim, self.kv_rank).transpose(1, 2).contiguous()
+        # per head (result index, summed index): uk transposed (it is applied to the query), uv as stored
+        self.uk = fetch(self._name("uk"), act, keep=False).view(H, self.dim, self.kv_rank).transpose(1, 2).contiguous()
+        self.uv = fetch(self._name("uv"), act).view(H, self.vdim, self.kv_rank).contiguous()
         self.out = LinearWeight(fetch(self._name("o"), act), self.precision)
         self.q_norm = fetch(self._name("dq.norm"))
         self.kv_norm = fetch(self._name("dkv.norm"))

@@ -351,18 +351,23 @@ def test_latent_prepare_kernel(dtype, q_rank, kv_rank, rot_dim, pairs):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("T,H,I,O", [(1, 3, 16, 40), (37, 5, 8, 24), (130, 2, 128, 300), (4, 16, 64, 512)])
+@pytest.mark.parametrize("T,H,I,O", [(1, 3, 16, 40), (37, 5, 8, 24), (130, 2, 128, 300), (4, 16, 64, 512), (70, 3, 96, 20),
+                                     (200, 2, 512, 128)])
 def test_headwise_linear_kernel(dtype, T, H, I, O):
     from qwen3_from_scratch_amd import ops
 
-    wide = _rand((T, H, I + 5), 1, dtype)
-    w = _rand((H, I, O), 2, dtype, I ** -0.5)
+    wide = _rand((T, H, I + 8), 1, dtype)          # rows that start at multiples of 16 bytes, as the model's do
+    w = _rand((H, O, I), 2, dtype, I ** -0.5)
     out = torch.zeros((T, H, O + 3), dtype=dtype).cuda()
     ops.headwise_linear(wide[:, :, :I], w, out=out[:, :, :O])          # both seen through strides
-    want = torch.einsum("thi,hio->tho", wide[:, :, :I].double(), w.double())
+    want = torch.einsum("thi,hoi->tho", wide[:, :, :I].double(), w.double())
     assert float((out[:, :, :O].double() - want).abs().max()) <= (1e-5 if dtype == torch.float32 else 3e-2)
     assert float(out[:, :, O:].abs().max()) == 0
     assert torch.equal(ops.headwise_linear(wide[:, :, :I].contiguous(), w), out[:, :, :O])
+    odd = _rand((T, H, I + 3), 1, dtype)            # and rows that do not: the multiply-add kernel
+    got = ops.headwise_linear(odd[:, :, 3:], w)
+    want = torch.einsum("thi,hoi->tho", odd[:, :, 3:].double(), w.double())
+    assert float((got.double() - want).abs().max()) <= (1e-5 if dtype == torch.float32 else 3e-2)
 
 
 @pytest.mark.gpu
@@ -405,9 +410,11 @@ def _paged(rows_per_seq, page, Dk, dtype, seed):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("general", [False, True])
 @pytest.mark.parametrize("H,Dk,Dv,page,window", [(3, 48, 40, 8, 19), (6, 160, 128, 16, 40), (5, 36, 24, 16, 0),
-                                                 (16, 96, 64, 32, 70), (2, 200, 136, 8, 1), (4, 576, 512, 16, 100)])
-def test_latent_attention_kernel(dtype, H, Dk, Dv, page, window):
+                                                 (16, 96, 64, 32, 70), (2, 200, 136, 8, 1), (4, 576, 512, 16, 100),
+                                                 (8, 288, 256, 16, 0), (7, 64, 16, 8, 33)])
+def test_latent_attention_kernel(dtype, H, Dk, Dv, page, window, general):
     """Prompts' portions beside single tokens, over scattered pages, against the twin; then
     queries made so that one key carries the whole softmax, that key just inside and just
     outside the window, at a page's first and last place, and far back without a window."""
@@ -421,7 +428,9 @@ def test_latent_attention_kernel(dtype, H, Dk, Dv, page, window):
     kvl = torch.tensor(kv, dtype=torch.int32).cuda()
     q = _rand((sum(q_lens), H, Dk), 3, dtype, 1.5)
     scale = Dk ** -0.5
-    a = ops.latent_attention(q, cache, Dv, table, cu, kvl, max(q_lens), scale, window=window)
+    if general and not (dtype == torch.bfloat16 and Dk % 32 == 0 and Dv % 16 == 0):
+        pytest.skip("these sizes take the general kernel anyway")
+    a = ops.latent_attention(q, cache, Dv, table, cu, kvl, max(q_lens), scale, window=window, general=general)
     b = torch_ops.latent_attention(q, cache, Dv, table, cu, kvl, max(q_lens), scale, window=window)
     assert a.shape == (sum(q_lens), H, Dv)
     assert float((a.float() - b.float()).abs().max()) <= (2e-5 if dtype == torch.float32 else 3e-2)
@@ -434,7 +443,8 @@ def test_latent_attention_kernel(dtype, H, Dk, Dv, page, window):
         peaked = q.clone()
         at = int(cu[seq]) + 1                           # the sequence's last token
         peaked[at] = (rows[seq][target] * 8.0).to(dtype).cuda()[None, :]
-        got = ops.latent_attention(peaked, cache, Dv, table, cu, kvl, max(q_lens), 1.0, window=window)[at].float()
+        got = ops.latent_attention(peaked, cache, Dv, table, cu, kvl, max(q_lens), 1.0, window=window,
+                                   general=general)[at].float()
         visible = window == 0 or back < window
         want = rows[seq][target, :Dv].float().cuda()
         close = float((got - want[None, :]).abs().max()) <= 0.05

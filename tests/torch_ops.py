@@ -241,7 +241,7 @@ def latent_prepare(down, q_rank, kv_rank, rot_dim, q_weight, kv_weight, eps, inv
 
 
 def headwise_linear(x, weight, out=None):
-    res = torch.einsum("thi,hio->tho", x.float(), weight.float()).to(x.dtype).contiguous()
+    res = torch.einsum("thi,hoi->tho", x.float(), weight.float()).to(x.dtype).contiguous()
     if out is not None:
         out.copy_(res)
         return out
@@ -253,7 +253,7 @@ def rotate_heads(x, out, inv_freq, rot_factor, positions):
     return out
 
 
-def latent_attention(q, cache, value_dim, block_table, cu_seqlens_q, kv_lens, max_q_len, scale, window=0):
+def latent_attention(q, cache, value_dim, block_table, cu_seqlens_q, kv_lens, max_q_len, scale, window=0, general=False):
     T, H, Dk = q.shape
     page = cache.shape[1]
     res = torch.zeros((T, H, value_dim), dtype=torch.float32, device=q.device)
