@@ -2,7 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--layers L]
                     [--shape 8b|14b|32b|0.6b] [--prompt P] [--context C]
-                    [--workload decode|continuous|served|prefix|products]
+                    [--workload decode|continuous|served|prefix|products|kodisun]
 
 Random bfloat16 weights, uniform-random prompts of 2,048 tokens, greedy decoding
 through the engine's own step loop (scheduler, step function, sampling). A
@@ -308,6 +308,116 @@ def shared_prefix(args, config, model, shape_name, gen, sync):
     return 0
 
 
+KODISUN_SHAPES = {
+    # (width, heads, dim, rot_dim, vdim, q_rank, kv_rank, window, experts, top, expert_ff, shared_ff, layers)
+    "lite": (2048, 16, 128, 64, 128, 768, 512, 1024, 64, 6, 1408, 2816, 4),
+    "mid": (4096, 32, 128, 64, 128, 1536, 512, 2048, 32, 4, 2048, 4096, 2),
+}
+
+
+def kodisun(args, sync):
+    """Prefill and decode throughput of the Kodisun design at sizes that resemble a real model's
+    layers (random weights, a few layers, a vocabulary of 32,768), beside the Qwen3 dense decoder
+    at equal size: the same width, head count and layer count, grouped heads of 128, and an inner
+    size equal to what a Kodisun token passes through (its chosen experts and the shared one).
+    Both go through the engine's own loop: one prompt of 2,048 tokens in one step, then greedy
+    decoding at batch 8 and 64 behind prompts of 1,024 tokens. `frac` prices a prompt's
+    multiply-adds against the bfloat16 matrix peak and a decode step's bytes (the weights it
+    touches once, the cached rows its requests see) against the HBM peak."""
+    import torch
+
+    from qwen3_from_scratch_amd.config import ModelConfig
+    from qwen3_from_scratch_amd.config.kodisun_config import KodisunConfig
+    from qwen3_from_scratch_amd.engine import SyncEngine, random_model
+
+    vocab, prompt_len, decode_prompt, context = 32768, args.prefill_tokens, 1024, 4096
+    results = {}
+    for shape in ([args.kodisun_shape] if args.kodisun_shape != "all" else sorted(KODISUN_SHAPES)):
+        W, H, dn, dr, dv, qr, kr, window, E, top, ff, sff, layers = KODISUN_SHAPES[shape]
+        if args.layers:
+            layers = args.layers
+        mixer = {"heads": H, "dim": dn, "rot_dim": dr, "vdim": dv, "q_rank": qr, "kv_rank": kr, "mask": {"size": window},
+                 "scale": (dn + dr) ** -0.5,
+                 "rot": {"dims": dr, "base": 10000.0, "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}
+        mlp = {"kind": "moe", "router": {"experts": E, "top": top}, "expert": {"ff": ff}, "shared": {"ff": sff}}
+        new = KodisunConfig.from_dict({"architecture": "Kodisun", "vocab": vocab, "width": W, "norm": {"eps": 1e-5},
+                                       "layers": [{"type": "latent_attention", "mixer": mixer, "mlp": mlp}] * layers})
+        dense = ModelConfig.from_dict(dict(QWEN3_8B, vocab_size=vocab, hidden_size=W, num_hidden_layers=layers,
+                                           num_attention_heads=H, num_key_value_heads=max(1, H // 4), head_dim=128,
+                                           intermediate_size=top * ff + sff, max_position_embeddings=context))
+        # what a token multiplies with, per layer, and what a decode step reads
+        new_active = ((qr + kr + dr) * W + H * (dn + dr) * qr + H * dn * kr + H * dv * kr + W * H * dv + E * W
+                      + 2 * top * ff * W + 2 * sff * W)
+        for name, config in (("kodisun", new), ("qwen3_dense", dense)):
+            if args.kodisun_only and name != args.kodisun_only:
+                continue
+            model = random_model(config, dtype=args.dtype, device="cuda:0", seed=0, std=0.02)
+            gen = torch.Generator().manual_seed(1)
+            entry = {}
+            if "prefill" in args.phases:
+                room = prompt_len + 64
+                engine = SyncEngine(model=model, path="", dtype=args.dtype, device="cuda:0", max_len=room, block_size=BLOCK,
+                                    num_blocks=-(-room // BLOCK), max_num_seqs=1, max_num_tokens=prompt_len,
+                                    chunked_prefill_size=prompt_len, enable_prefix_cache=False)
+                timings = []
+                for _ in range(4):
+                    engine.add_request(torch.randint(0, vocab, (prompt_len,), generator=gen).tolist(),
+                                       engine.default_params(1, temperature=0.0, ignore_eos=True))
+                    sync()
+                    t0 = time.perf_counter()
+                    engine.step()
+                    sync()
+                    timings.append(time.perf_counter() - t0)
+                    while engine.scheduler.has_work():
+                        engine.step()
+                seconds = sorted(timings[1:])[1]
+                if name == "kodisun":
+                    pairs = sum(min(i + 1, window) for i in range(prompt_len))
+                    flops = layers * (2.0 * prompt_len * new_active + 2.0 * pairs * H * ((kr + dr) + kr)) + 2.0 * prompt_len * vocab * W
+                else:
+                    flops = prefill_flops(config, prompt_len)
+                entry["prefill"] = {"tokens": prompt_len, "tokens_per_s": round(prompt_len / seconds, 1),
+                                    "ms": round(seconds * 1e3, 3), "frac": round(flops / seconds / PEAK_FLOPS[args.dtype], 4)}
+                del engine
+            for batch in ((8, 64) if "decode" in args.phases else ()):
+                engine = SyncEngine(model=model, path="", dtype=args.dtype, device="cuda:0", max_len=context,
+                                    block_size=BLOCK, num_blocks=batch * (context // BLOCK), max_num_seqs=batch,
+                                    max_num_tokens=max(2048, batch), chunked_prefill_size=2048, enable_prefix_cache=False)
+                params = engine.default_params(context - decode_prompt - 1, temperature=0.0, ignore_eos=True)
+                requests = [engine.add_request(torch.randint(0, vocab, (decode_prompt,), generator=gen).tolist(), params)
+                            for _ in range(batch)]
+                while any(r.is_prefill for r in requests) or len(engine.scheduler.waiting):
+                    engine.step()
+                for _ in range(args.warmup):
+                    engine.step()
+                sync()
+                t0 = time.perf_counter()
+                for _ in range(args.steps):
+                    engine.step()
+                sync()
+                step_s = (time.perf_counter() - t0) / args.steps
+                seen = decode_prompt + args.warmup + args.steps // 2
+                if name == "kodisun":
+                    touched = min(E, batch * top)                      # experts a step can touch at most
+                    weights = layers * (new_active - 2 * top * ff * W + 2 * touched * ff * W) + vocab * W
+                    need = 2 * (weights + layers * batch * min(seen, window) * (kr + dr))
+                else:
+                    need = decode_bytes(config, [seen] * batch, 2)
+                entry["decode_b%d" % batch] = {"tokens_per_s": round(batch / step_s, 1), "ms_per_step": round(step_s * 1e3, 3),
+                                               "frac_hbm": round(need / step_s / PEAK_HBM, 4)}
+                del engine
+            results.setdefault(shape, {})[name] = entry
+            del model
+            torch.cuda.empty_cache()
+        results[shape]["sizes"] = {"width": W, "heads": H, "dim": dn, "rot_dim": dr, "vdim": dv, "q_rank": qr, "kv_rank": kr,
+                                   "window": window, "experts": E, "top": top, "expert_ff": ff, "shared_ff": sff,
+                                   "layers": layers, "dense_intermediate": top * ff + sff, "vocab": vocab}
+    print(json.dumps({"metric": "Kodisun beside the Qwen3 dense decoder at equal size: prefill and decode tokens/s",
+                      "unit": "tokens/s", "n_gpus": 1, "higher_is_better": True, "dtype": "bf16", "data": "synthetic",
+                      "steps": args.steps, "warmup": args.warmup, "shapes": results}))
+    return 0
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -319,12 +429,15 @@ def main():
     ap.add_argument("--shape", default="8b", choices=sorted(SHAPES))
     ap.add_argument("--prompt", type=int, default=2048, help="tokens every request holds when decoding starts")
     ap.add_argument("--context", type=int, default=8192, help="tokens of cache per request")
-    ap.add_argument("--workload", default="decode", choices=["decode", "continuous", "served", "prefix", "products"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "continuous", "served", "prefix", "products", "kodisun"],
                     help="continuous: 64 requests at once, prompts of 128 to 4,096 tokens, 64 to 512 generated "
                          "tokens each, prompts in portions of 512 (its own JSON line; --steps and --warmup unused); "
                          "prefix: 64 requests that share their first 2,048 tokens, with the prefix index on and off; "
                          "products: a layer's four products by the chosen kernel and by each tile shape of the "
-                         "hand-written one")
+                         "hand-written one; kodisun: the Kodisun design beside the dense decoder at equal size")
+    ap.add_argument("--kodisun-shape", default="all", choices=["all"] + sorted(KODISUN_SHAPES))
+    ap.add_argument("--kodisun-only", default="", choices=["", "kodisun", "qwen3_dense"], help="one of the two models")
+    ap.add_argument("--phases", default="prefill,decode", help="of --workload kodisun: prefill, decode or both")
     ap.add_argument("--single-copy", action="store_true",
                     help="hold the matrices once (no tile-ordered copy for steps of few rows): half the weights' memory, slower decoding")
     ap.add_argument("--no-points", action="store_true", help="skip the batch-1 and batch-64 points")
@@ -344,6 +457,10 @@ def main():
     from qwen3_from_scratch_amd.config import ModelConfig
     from qwen3_from_scratch_amd.engine import SyncEngine, random_model
 
+    if args.workload == "kodisun":
+        torch.cuda.set_device(0)
+        args.steps, args.warmup = min(args.steps, 32), min(args.warmup, 8)
+        return kodisun(args, torch.cuda.synchronize)
     shape_name, raw = SHAPES[args.shape]
     raw = dict(raw)
     prompt_len, context = args.prompt, args.context

@@ -26,7 +26,7 @@ def main(argv=None):
     parser.add_argument("--max-tokens", type=int, required=True,
                         help="most tokens live requests hold at any time (each rounded up to 64)")
     parser.add_argument("--page-size", type=int, default=16)
-    parser.add_argument("--max-requests", type=int, default=8)
+    parser.add_argument("--max-requests", type=int, default=4, help="requests that are live at any time")
     args = parser.parse_args(argv)
 
     import numpy as np
