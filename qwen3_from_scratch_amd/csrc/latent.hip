@@ -341,20 +341,41 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(const T* __restrict__ 
 #define LMA_KPAD 8
 #define LMA_VLD 40   // halfwords per transposed row: 32 keys and 8 of padding
 
+// Which sequence and which of its row tiles a block serves: blocks are numbered through the
+// sequences' tiles of 64 rows in turn (a step's sequences bring very different numbers of rows, and
+// a grid of the longest's tiles for every sequence would be mostly blocks that start and end).
+__device__ inline bool lma_find_tile(const int* __restrict__ cu_q, int B, int H, int tile, int& b, int& m0) {
+  int at = 0;
+  for (int i = 0; i < B; ++i) {
+    const int n = ((cu_q[i + 1] - cu_q[i]) * H + LMA_ROWS - 1) / LMA_ROWS;
+    if (tile < at + n) {
+      b = i;
+      m0 = (tile - at) * LMA_ROWS;
+      return true;
+    }
+    at += n;
+  }
+  return false;
+}
+
+// KS: most steps of 32 over Dk; NV: most slabs of 16 over Dv. With `splits` > 1 (blockIdx.y) a
+// block walks its share of the tiles and leaves float32 sums that are not yet divided, with the
+// row's maximum (in the exponent's units) and sum, in `partial` ((rows, splits, Dv + 2) floats,
+// rows numbered (packed token, head)); `latent_attn_merge_kernel` joins the shares in their order.
 template <int KS, int NV>
 __global__ __launch_bounds__(256) void latent_attn_mma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
                                                               const bf16_t* __restrict__ cache, int num_pages,
                                                               const int* __restrict__ block_table, int bt_stride,
                                                               const int* __restrict__ cu_q,
-                                                              const int* __restrict__ kv_lens, int H, int Dk, int Dv,
-                                                              int page, float scale_log2, int window) {
+                                                              const int* __restrict__ kv_lens, int B, int H, int Dk,
+                                                              int Dv, int page, float scale_log2, int window,
+                                                              int splits, float* __restrict__ partial) {
   extern __shared__ __align__(16) unsigned char lma_smem[];
-  const int b = blockIdx.y;
+  int b, m0;
+  if (!lma_find_tile(cu_q, B, H, blockIdx.x, b, m0)) return;
   const int q0 = cu_q[b];
   const int q_len = cu_q[b + 1] - q0;
   const int n_rows = q_len * H;
-  const int m0 = blockIdx.x * LMA_ROWS;
-  if (m0 >= n_rows) return;
   const int kv_len = kv_lens[b];
   const int base_pos = kv_len - q_len;
   const int ldk = Dk + LMA_KPAD;                              // halfwords per key row
@@ -364,11 +385,18 @@ __global__ __launch_bounds__(256) void latent_attn_mma_kernel(const bf16_t* __re
   const int col = lane & 15, grp = lane >> 4;
   const int ks = Dk >> 5, nv = Dv >> 4;
 
-  // the block's span of keys, and this wavefront's
+  // the block's span of keys (and of that this block's share), and this wavefront's
   const int block_last = min(m0 + LMA_ROWS, n_rows) - 1;
-  const int k_end = base_pos + block_last / H + 1;
+  int k_end = base_pos + block_last / H + 1;
   int k_begin = window > 0 ? max(0, base_pos + m0 / H - window + 1) : 0;
   k_begin -= k_begin % LMA_BN;
+  if (splits > 1) {
+    const int tiles = (k_end - k_begin + LMA_BN - 1) / LMA_BN;
+    const int share = (tiles + splits - 1) / splits;
+    const int first = k_begin + blockIdx.y * share * LMA_BN;
+    k_end = min(k_end, first + share * LMA_BN);
+    k_begin = first;
+  }
   const int w0 = m0 + 16 * wave;
   const bool wave_active = w0 < n_rows;
   const int wave_last = min(w0 + 16, n_rows) - 1;
@@ -393,27 +421,50 @@ __global__ __launch_bounds__(256) void latent_attn_mma_kernel(const bf16_t* __re
   float m_run = -INFINITY, l_run = 0.f;
   const int chunks_per_key = Dk >> 3;
   const int chunks = LMA_BN * chunks_per_key;
+  constexpr int NCH = (KS + 1) / 2;                           // 16-byte pieces of a tile per thread
+  uint4 pre[NCH];
 
-  for (int kt0 = k_begin; kt0 < k_end; kt0 += LMA_BN) {
-    __syncthreads();
-    for (int c = threadIdx.x; c < chunks; c += 256) {
-      const int j = c / chunks_per_key, d0 = (c - j * chunks_per_key) * 8;
-      const int kj = kt0 + j;
-      LatPack v;
-      v.u = make_uint4(0, 0, 0, 0);
-      if (kj < k_end) {
-        const int pg = block_table[(size_t)b * bt_stride + kj / page];
-        if (pg >= 0 && pg < num_pages)
-          v.u = *reinterpret_cast<const uint4*>(cache + ((size_t)pg * page + kj % page) * Dk + d0);
-      }
-      *reinterpret_cast<uint4*>(kt + j * ldk + d0) = v.u;
-      if (d0 < Dv) {
-        const unsigned short* e = reinterpret_cast<const unsigned short*>(&v.u);
-        unsigned short* dst = reinterpret_cast<unsigned short*>(vt) + d0 * LMA_VLD + j;
+  // a tile's pieces on their way from the cache into registers
+  auto fetch = [&](int kt0) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) dst[i * LMA_VLD] = e[i];
+    for (int i = 0; i < NCH; ++i) {
+      const int c = threadIdx.x + 256 * i;
+      pre[i] = make_uint4(0, 0, 0, 0);
+      if (c < chunks) {
+        const int j = c / chunks_per_key, d0 = (c - j * chunks_per_key) * 8;
+        const int kj = kt0 + j;
+        if (kj < k_end) {
+          const int pg = block_table[(size_t)b * bt_stride + kj / page];
+          if (pg >= 0 && pg < num_pages)
+            pre[i] = *reinterpret_cast<const uint4*>(cache + ((size_t)pg * page + kj % page) * Dk + d0);
+        }
       }
     }
+  };
+
+  if (k_begin < k_end) fetch(k_begin);
+  for (int kt0 = k_begin; kt0 < k_end; kt0 += LMA_BN) {
+    __syncthreads();                                          // the last tile's readers are done
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      const int c = threadIdx.x + 256 * i;
+      if (c < chunks) {
+        const int j = c / chunks_per_key, d0 = (c - j * chunks_per_key) * 8;
+        *reinterpret_cast<uint4*>(kt + j * ldk + d0) = pre[i];
+      }
+    }
+    __syncthreads();
+    // the values' copy: lanes side by side take keys side by side, so that they write runs of a transposed row
+    for (int item = threadIdx.x; item < LMA_BN * (Dv >> 3); item += 256) {
+      const int j = item & (LMA_BN - 1), d0 = (item >> 5) * 8;
+      LatPack v;
+      v.u = *reinterpret_cast<const uint4*>(kt + j * ldk + d0);
+      unsigned short* dst = reinterpret_cast<unsigned short*>(vt) + d0 * LMA_VLD + j;
+      const unsigned short* e = reinterpret_cast<const unsigned short*>(&v.u);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) dst[i * LMA_VLD] = e[i];
+    }
+    if (kt0 + LMA_BN < k_end) fetch(kt0 + LMA_BN);            // the next tile travels while this one is worked on
     __syncthreads();
     if (!wave_active || kt0 >= wave_k_end || kt0 + LMA_BN <= wave_k_begin) continue;
     lat_f32x4_t sc[2];
@@ -435,7 +486,7 @@ __global__ __launch_bounds__(256) void latent_attn_mma_kernel(const bf16_t* __re
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       const int key = kt0 + 16 * (j >> 2) + 4 * grp + (j & 3);
-      bool seen = valid && key <= pos;
+      bool seen = valid && key <= pos && key < k_end;
       if (window > 0 && pos - key >= window) seen = false;
       v[j] = seen ? sc[j >> 2][j & 3] : -INFINITY;
     }
@@ -471,21 +522,54 @@ __global__ __launch_bounds__(256) void latent_attn_mma_kernel(const bf16_t* __re
       }
     }
   }
-  if (valid) {
-    const float inv = 1.f / l_run;
-    bf16_t* o = out + ((size_t)(q0 + tok) * H + head) * Dv + 4 * grp;
+  if (!valid) return;
+  if (splits > 1) {
+    float* dst = partial + (((size_t)(q0 + tok) * H + head) * splits + blockIdx.y) * (Dv + 2);
+    if (grp == 0) {
+      dst[Dv] = m_run;
+      dst[Dv + 1] = l_run;
+    }
 #pragma unroll
     for (int nb = 0; nb < NV; ++nb) {
-      if (nb < nv) {
-        union {
-          uint2 u;
-          bf16_t e[4];
-        } pk;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) pk.e[i] = float_to_bf16(acc[nb][i] * inv);
-        *reinterpret_cast<uint2*>(o + 16 * nb) = pk.u;
-      }
+      if (nb < nv) *reinterpret_cast<float4*>(dst + 16 * nb + 4 * grp) = make_float4(acc[nb][0], acc[nb][1], acc[nb][2], acc[nb][3]);
     }
+    return;
+  }
+  const float inv = 1.f / l_run;
+  bf16_t* o = out + ((size_t)(q0 + tok) * H + head) * Dv + 4 * grp;
+#pragma unroll
+  for (int nb = 0; nb < NV; ++nb) {
+    if (nb < nv) {
+      union {
+        uint2 u;
+        bf16_t e[4];
+      } pk;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) pk.e[i] = float_to_bf16(acc[nb][i] * inv);
+      *reinterpret_cast<uint2*>(o + 16 * nb) = pk.u;
+    }
+  }
+}
+
+// out[row] = sum_s 2^(m_s - m) acc_s / sum_s 2^(m_s - m) l_s, m = max_s m_s, the shares in their order.
+__global__ void latent_attn_merge_kernel(const float* __restrict__ partial, bf16_t* __restrict__ out, int Dv, int splits) {
+  const size_t row = blockIdx.x;
+  const float* src = partial + row * splits * (Dv + 2);
+  float m = -INFINITY;
+  for (int s = 0; s < splits; ++s) m = fmaxf(m, src[(size_t)s * (Dv + 2) + Dv]);
+  float l = 0.f;
+  for (int s = 0; s < splits; ++s) {
+    const float ms = src[(size_t)s * (Dv + 2) + Dv];
+    if (ms > -INFINITY) l += exp2f(ms - m) * src[(size_t)s * (Dv + 2) + Dv + 1];
+  }
+  const float inv = 1.f / l;
+  for (int d = threadIdx.x; d < Dv; d += blockDim.x) {
+    float a = 0.f;
+    for (int s = 0; s < splits; ++s) {
+      const float ms = src[(size_t)s * (Dv + 2) + Dv];
+      if (ms > -INFINITY) a += exp2f(ms - m) * src[(size_t)s * (Dv + 2) + d];
+    }
+    out[row * Dv + d] = float_to_bf16(a * inv);
   }
 }
 
@@ -581,16 +665,20 @@ static int launch_latent_attn(const void* q, void* out, const void* cache, int n
 
 template <int KS, int NV>
 static int launch_latent_attn_mma(const void* q, void* out, const void* cache, int num_pages, const int* block_table,
-                                  int bt_stride, const int* cu_q, const int* kv_lens, int B, int H, int Dk, int Dv,
-                                  int page, float scale, int window, int max_q_len, hipStream_t stream) {
+                                  int bt_stride, const int* cu_q, const int* kv_lens, int B, int T, int H, int Dk,
+                                  int Dv, int page, float scale, int window, int splits, float* partial,
+                                  hipStream_t stream) {
   const size_t smem = (size_t)(LMA_BN * (Dk + LMA_KPAD) + Dv * LMA_VLD) * sizeof(bf16_t);
   int e = raise_shared_memory((const void*)latent_attn_mma_kernel<KS, NV>, smem);
   if (e) return e;
-  const long tiles = ((long)max_q_len * H + LMA_ROWS - 1) / LMA_ROWS;
-  if (tiles > 0x7fffffffL || B > 65535) return Q3_ERR_UNSUPPORTED;
-  hipLaunchKernelGGL((latent_attn_mma_kernel<KS, NV>), dim3((unsigned)tiles, B), dim3(256), smem, stream,
+  const long tiles = ((long)T * H) / LMA_ROWS + B;            // at least the sequences' tiles of 64 rows together
+  if (tiles > 0x7fffffffL || splits < 1 || splits > 65535 || (splits > 1 && !partial)) return Q3_ERR_UNSUPPORTED;
+  hipLaunchKernelGGL((latent_attn_mma_kernel<KS, NV>), dim3((unsigned)tiles, splits), dim3(256), smem, stream,
                      (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)cache, num_pages, block_table, bt_stride, cu_q,
-                     kv_lens, H, Dk, Dv, page, scale * 1.44269504088896341f, window);
+                     kv_lens, B, H, Dk, Dv, page, scale * 1.44269504088896341f, window, splits, partial);
+  if (splits > 1)
+    hipLaunchKernelGGL(latent_attn_merge_kernel, dim3((unsigned)((long)T * H)), dim3(Dv >= 256 ? 256 : 64), 0, stream,
+                       partial, (bf16_t*)out, Dv, splits);
   return q3_launch_status();
 }
 
@@ -600,21 +688,21 @@ extern "C" int q3_latent_attention_fast_path(int Dk, int Dv, int dtype) {
 }
 
 extern "C" int q3_latent_attention(const void* q, void* out, const void* cache, int num_pages, const int* block_table,
-                                   int bt_stride, const int* cu_q, const int* kv_lens, int B, int H, int Dk, int Dv,
-                                   int page, float scale, int window, int max_q_len, int dtype, int general,
-                                   hipStream_t stream) {
-  if (B <= 0 || H <= 0 || Dk <= 0 || Dv <= 0 || Dv > Dk || page <= 0 || max_q_len <= 0 || window < 0)
+                                   int bt_stride, const int* cu_q, const int* kv_lens, int B, int T, int H, int Dk,
+                                   int Dv, int page, float scale, int window, int max_q_len, int dtype, int general,
+                                   int splits, float* partial, hipStream_t stream) {
+  if (B <= 0 || T <= 0 || H <= 0 || Dk <= 0 || Dv <= 0 || Dv > Dk || page <= 0 || max_q_len <= 0 || window < 0)
     return Q3_ERR_BAD_ARGUMENT;
   if (Dv > 1024) return Q3_ERR_UNSUPPORTED;
   if (!general && q3_latent_attention_fast_path(Dk, Dv, dtype)) {
     if (Dk <= 192 && Dv <= 128)
-      return launch_latent_attn_mma<6, 8>(q, out, cache, num_pages, block_table, bt_stride, cu_q, kv_lens, B, H, Dk, Dv,
-                                          page, scale, window, max_q_len, stream);
+      return launch_latent_attn_mma<6, 8>(q, out, cache, num_pages, block_table, bt_stride, cu_q, kv_lens, B, T, H, Dk,
+                                          Dv, page, scale, window, splits, partial, stream);
     if (Dk <= 320 && Dv <= 256)
-      return launch_latent_attn_mma<10, 16>(q, out, cache, num_pages, block_table, bt_stride, cu_q, kv_lens, B, H, Dk,
-                                            Dv, page, scale, window, max_q_len, stream);
-    return launch_latent_attn_mma<18, 32>(q, out, cache, num_pages, block_table, bt_stride, cu_q, kv_lens, B, H, Dk, Dv,
-                                          page, scale, window, max_q_len, stream);
+      return launch_latent_attn_mma<10, 16>(q, out, cache, num_pages, block_table, bt_stride, cu_q, kv_lens, B, T, H,
+                                            Dk, Dv, page, scale, window, splits, partial, stream);
+    return launch_latent_attn_mma<18, 32>(q, out, cache, num_pages, block_table, bt_stride, cu_q, kv_lens, B, T, H, Dk,
+                                          Dv, page, scale, window, splits, partial, stream);
   }
   Q3_DISPATCH_DTYPE(dtype, TT, {
     if (Dv <= 128)

@@ -11,36 +11,27 @@ __device__ inline float moe_gelu(float z, int kind) {
 }
 
 // ---------------------------------------------------------------------------
-// The router. One wavefront per token: z_e = router[e] . h (float32 sums over bfloat16 or float32
-// numbers), s = softmax(z) over all E experts, then `top` times the largest remaining score (the
-// lowest index among equals); weight_k = s_k / (sum of the chosen s + 1e-20).
+// The router's choice. One wavefront per token, from its float32 logits z (E numbers):
+// s = softmax(z) over all E experts, then `top` times the largest remaining score (the lowest
+// index among equals); weight_k = s_k / (sum of the chosen s + 1e-20). Every lane holds every
+// reduced number and writes the same value to the same place of shared memory, so nothing here
+// waits for another lane's write.
 // ---------------------------------------------------------------------------
-template <typename T>
-__global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ h, const T* __restrict__ router,
-                                                        int n_tokens, int width, int E, int top,
-                                                        int* __restrict__ chosen, float* __restrict__ weights) {
+__global__ __launch_bounds__(256) void moe_pick_kernel(const float* __restrict__ logits, int n_tokens, int E, int top,
+                                                       int* __restrict__ chosen, float* __restrict__ weights) {
   extern __shared__ float smem[];
   const int wave = threadIdx.x / Q3_WAVE, lane = threadIdx.x % Q3_WAVE;
   const int t = blockIdx.x * (blockDim.x / Q3_WAVE) + wave;
   if (t >= n_tokens) return;
   float* z = smem + (size_t)wave * (E + top);     // the wavefront's scores, then the chosen ones
   float* picked = z + E;
-  const T* x = h + (size_t)t * width;
-  // every lane holds every sum after the butterfly and writes the same number to the same place,
-  // so nothing here waits for another lane's write
-  for (int e = 0; e < E; ++e) {
-    const T* w = router + (size_t)e * width;
-    float acc = 0.f;
-    for (int j = lane; j < width; j += Q3_WAVE) acc += to_float(x[j]) * to_float(w[j]);
-    z[e] = wave_sum(acc);
-  }
-  __builtin_amdgcn_wave_barrier();
+  const float* src = logits + (size_t)t * E;
   float biggest = -INFINITY;
-  for (int e = lane; e < E; e += Q3_WAVE) biggest = fmaxf(biggest, z[e]);
+  for (int e = lane; e < E; e += Q3_WAVE) biggest = fmaxf(biggest, src[e]);
   biggest = wave_max(biggest);
   float total = 0.f;
   for (int e = lane; e < E; e += Q3_WAVE) {
-    const float p = expf(z[e] - biggest);
+    const float p = expf(src[e] - biggest);
     z[e] = p;
     total += p;
   }
@@ -189,9 +180,10 @@ __global__ __launch_bounds__(256) void moe_linear_kernel(const T* __restrict__ x
 // The same products on the matrix cores (v_mfma_f32_16x16x32_bf16): bfloat16, K a multiple of 32.
 // out^T (columns x slots) = W_e (columns x K) . x^T (K x slots): 16 weight rows are the first
 // operand, 16 slots' rows of x the second, both straight from memory (a lane reads 16 bytes of
-// one row per step of 32 k). A tile has 32 slots (two second operands); a block's four wavefronts
-// each own NS slabs of 16 output columns, so every x operand serves NS matrix instructions and
-// every weight operand two. A lane ends up with four consecutive columns of one slot.
+// one row per step of 32 k). A tile has up to 64 slots (four second operands, of which those
+// beyond the tile's rows are skipped); a block's four wavefronts each own NS slabs of 16 output
+// columns, so every x operand serves NS matrix instructions and every weight operand up to four.
+// A lane ends up with four consecutive columns of one slot.
 // ---------------------------------------------------------------------------
 typedef __attribute__((ext_vector_type(8))) __bf16 moe_bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) float moe_f32x4_t;
@@ -199,7 +191,8 @@ union MoePack {
   uint4 u;
   moe_bf16x8_t v;
 };
-#define MMA_TM 32
+#define MMA_TM 64
+#define MMA_MT 4
 
 template <int NS>
 __global__ __launch_bounds__(256) void moe_linear_mma_kernel(
@@ -214,9 +207,9 @@ __global__ __launch_bounds__(256) void moe_linear_mma_kernel(
   const int rows = min(MMA_TM, offsets[e + 1] - first);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int col = lane & 15, grp = lane >> 4;
-  const bf16_t* xr[2];
+  const bf16_t* xr[MMA_MT];
 #pragma unroll
-  for (int mt = 0; mt < 2; ++mt) {
+  for (int mt = 0; mt < MMA_MT; ++mt) {
     const int m = 16 * mt + col;
     xr[mt] = nullptr;
     if (m < rows) {
@@ -232,29 +225,32 @@ __global__ __launch_bounds__(256) void moe_linear_mma_kernel(
     const int n = n_base + 16 * ns + col;
     wr[ns] = n < N ? w + ((size_t)e * N + n) * K + 8 * grp : nullptr;
   }
-  moe_f32x4_t acc[2][NS];
+  moe_f32x4_t acc[MMA_MT][NS];
 #pragma unroll
-  for (int mt = 0; mt < 2; ++mt)
+  for (int mt = 0; mt < MMA_MT; ++mt)
 #pragma unroll
     for (int ns = 0; ns < NS; ++ns) acc[mt][ns] = moe_f32x4_t{0.f, 0.f, 0.f, 0.f};
-  const bool two = rows > 16;
-#pragma unroll 4
+  const int row_blocks = (rows + 15) >> 4;          // the same for every lane
+#pragma unroll 2
   for (int k0 = 0; k0 < K; k0 += 32) {
-    MoePack a[NS], b[2];
+    MoePack a[NS], b[MMA_MT];
 #pragma unroll
     for (int ns = 0; ns < NS; ++ns)
       a[ns].u = wr[ns] ? *reinterpret_cast<const uint4*>(wr[ns] + k0) : make_uint4(0, 0, 0, 0);
 #pragma unroll
-    for (int mt = 0; mt < 2; ++mt)
-      b[mt].u = xr[mt] ? *reinterpret_cast<const uint4*>(xr[mt] + k0) : make_uint4(0, 0, 0, 0);
+    for (int mt = 0; mt < MMA_MT; ++mt)
+      b[mt].u = (mt < row_blocks && xr[mt]) ? *reinterpret_cast<const uint4*>(xr[mt] + k0) : make_uint4(0, 0, 0, 0);
 #pragma unroll
-    for (int ns = 0; ns < NS; ++ns) {
-      acc[0][ns] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[ns].v, b[0].v, acc[0][ns], 0, 0, 0);
-      if (two) acc[1][ns] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[ns].v, b[1].v, acc[1][ns], 0, 0, 0);
+    for (int mt = 0; mt < MMA_MT; ++mt) {
+      if (mt < row_blocks) {
+#pragma unroll
+        for (int ns = 0; ns < NS; ++ns)
+          acc[mt][ns] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[ns].v, b[mt].v, acc[mt][ns], 0, 0, 0);
+      }
     }
   }
 #pragma unroll
-  for (int mt = 0; mt < 2; ++mt) {
+  for (int mt = 0; mt < MMA_MT; ++mt) {
     const int m = 16 * mt + col;
     if (m >= rows) continue;
 #pragma unroll
@@ -290,19 +286,17 @@ __global__ void moe_combine_kernel(const T* __restrict__ y, const int* __restric
   }
 }
 
-extern "C" int q3_moe_route(const void* h, const void* router, int n_tokens, int width, int E, int top, int* chosen,
-                            float* weights, int dtype, hipStream_t stream) {
-  if (n_tokens <= 0 || width <= 0 || E <= 0 || top <= 0 || top > E || E > 4096) return Q3_ERR_BAD_ARGUMENT;
+extern "C" int q3_moe_pick(const float* logits, int n_tokens, int E, int top, int* chosen, float* weights,
+                           hipStream_t stream) {
+  if (n_tokens <= 0 || E <= 0 || top <= 0 || top > E || E > 4096) return Q3_ERR_BAD_ARGUMENT;
   const int waves = 4;
   const size_t smem = (size_t)waves * (E + top) * sizeof(float);
-  Q3_DISPATCH_DTYPE(dtype, TT,
-                    hipLaunchKernelGGL(moe_route_kernel<TT>, dim3((n_tokens + waves - 1) / waves), dim3(waves * Q3_WAVE),
-                                       smem, stream, (const TT*)h, (const TT*)router, n_tokens, width, E, top, chosen,
-                                       weights));
+  hipLaunchKernelGGL(moe_pick_kernel, dim3((n_tokens + waves - 1) / waves), dim3(waves * Q3_WAVE), smem, stream, logits,
+                     n_tokens, E, top, chosen, weights);
   return q3_launch_status();
 }
 
-// Slots per tile: 16 for the float32 multiply-add kernel, 32 for the matrix-core kernel.
+// Slots per tile: 16 for the float32 multiply-add kernel, 64 for the matrix-core kernel.
 extern "C" int q3_moe_tile_rows(int matrix_cores) { return matrix_cores ? MMA_TM : MOE_BM; }
 
 extern "C" int q3_moe_align(const int* chosen, int P, int E, int tile_rows, int* offsets, int* pair_of_slot,
@@ -313,22 +307,22 @@ extern "C" int q3_moe_align(const int* chosen, int P, int E, int tile_rows, int*
   return q3_launch_status();
 }
 
-// The matrix-core product: bfloat16, K a multiple of 32, tiles of 32 slots.
+// The matrix-core product: bfloat16, K a multiple of 32, tiles of 64 slots.
 extern "C" int q3_moe_linear_mma(const void* x, const int* pair_of_slot, int gather, int pairs_per_row, const void* w,
                                  void* out, const int* tile_expert, const int* tile_first, const int* offsets,
                                  const int* n_tiles, int max_tiles, int N, int K, int act, hipStream_t stream) {
   if (max_tiles <= 0 || N <= 0 || K <= 0 || K % 32 || pairs_per_row <= 0 || act < -1 || act > 1)
     return Q3_ERR_BAD_ARGUMENT;
   // few blocks (steps of few tokens): one slab of 16 columns per wavefront, so that more blocks stream the weights
-  const bool narrow = (long)max_tiles * ((N + 127) / 128) < 512;
-  const int per_block = narrow ? 64 : 128;
+  const bool narrow = (long)max_tiles * ((N + 255) / 256) < 512;
+  const int per_block = narrow ? 64 : 256;
   const dim3 grid(max_tiles, (N + per_block - 1) / per_block);
   if (grid.y > 65535) return Q3_ERR_UNSUPPORTED;
   if (narrow)
     hipLaunchKernelGGL(moe_linear_mma_kernel<1>, grid, dim3(256), 0, stream, (const bf16_t*)x, pair_of_slot, gather,
                        pairs_per_row, (const bf16_t*)w, (bf16_t*)out, tile_expert, tile_first, offsets, n_tiles, N, K, act);
   else
-    hipLaunchKernelGGL(moe_linear_mma_kernel<2>, grid, dim3(256), 0, stream, (const bf16_t*)x, pair_of_slot, gather,
+    hipLaunchKernelGGL(moe_linear_mma_kernel<4>, grid, dim3(256), 0, stream, (const bf16_t*)x, pair_of_slot, gather,
                        pairs_per_row, (const bf16_t*)w, (bf16_t*)out, tile_expert, tile_first, offsets, n_tiles, N, K, act);
   return q3_launch_status();
 }

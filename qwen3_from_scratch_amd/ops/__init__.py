@@ -438,7 +438,7 @@ def rotate_heads(x, out, inv_freq, rot_factor, positions):
 
 
 def latent_attention(q, cache, value_dim, block_table, cu_seqlens_q, kv_lens, max_q_len, scale, window=0,
-                     general=False):
+                     general=False, max_kv_len=0):
     """Causal softmax attention of every head's query rows over one shared sequence of cached rows.
 
     q (T, H, Dk) contiguous; cache (pages, page, Dk): the row of sequence b's position j lies in
@@ -447,7 +447,9 @@ def latent_attention(q, cache, value_dim, block_table, cu_seqlens_q, kv_lens, ma
     positions j <= its own and, with window > 0, only those fewer than `window` behind it.
     Returns (T, H, value_dim). Float32 scores, statistics and sums. bfloat16 with Dk in steps of 32
     (up to 576) and value_dim in steps of 16 (up to 512) runs on the matrix cores; everything
-    else, and everything with `general=True`, takes the kernel of float32 multiply-adds."""
+    else, and everything with `general=True`, takes the kernel of float32 multiply-adds.
+    `max_q_len` bounds the sequences' rows and `max_kv_len` (0: unknown) their keys: a step of few
+    rows over many keys shares the keys out over several blocks per row tile."""
     _dev(q, cache, block_table, cu_seqlens_q, kv_lens)
     _need(q.dim() == 3 and q.dtype in _DT and cache.dim() == 3 and cache.dtype == q.dtype
           and cache.shape[2] == q.shape[2], "q (T, H, Dk) and cache (pages, page, Dk) of one dtype")
@@ -460,18 +462,36 @@ def latent_attention(q, cache, value_dim, block_table, cu_seqlens_q, kv_lens, ma
           "block_table must be int32 (B, W)")
     out = torch.empty((T, H, value_dim), dtype=q.dtype, device=q.device)
     if T and B:
-        _check(library("latent").q3_latent_attention(
+        lib = library("latent")
+        splits, partial = 1, None
+        if not general and lib.q3_latent_attention_fast_path(Dk, value_dim, _DT[q.dtype]):
+            splits = _latent_splits(T, B, H, max_q_len, max_kv_len, window)
+            if splits > 1:
+                partial = torch.empty((T * H * splits * (value_dim + 2),), dtype=torch.float32, device=q.device)
+        _check(lib.q3_latent_attention(
             _ptr(q), _ptr(out), _ptr(cache), cache.shape[0], _ptr(block_table), block_table.shape[1],
-            _ptr(cu_seqlens_q), _ptr(kv_lens), B, H, Dk, value_dim, cache.shape[1], ctypes.c_float(scale), int(window),
-            int(max_q_len), _DT[q.dtype], 1 if general else 0, _stream()), "latent_attention")
+            _ptr(cu_seqlens_q), _ptr(kv_lens), B, T, H, Dk, value_dim, cache.shape[1], ctypes.c_float(scale), int(window),
+            int(max_q_len), _DT[q.dtype], 1 if general else 0, splits, _ptr(partial), _stream()), "latent_attention")
     return out
 
 
-def moe_route(h, router, top):
+def _latent_splits(T, B, H, max_q_len, max_kv_len, window):
+    """Over how many blocks a row tile's keys are shared out: only where the step's row tiles
+    (64 rows each) leave most of the chip idle and there are keys enough, at least four tiles of
+    32 to a share, until there are two blocks a compute unit."""
+    tiles = (T * H) // 64 + B
+    keys = max_kv_len if window <= 0 else min(max_kv_len, window + max_q_len)
+    if tiles >= 256 or keys < 256:
+        return 1
+    return max(1, min(512 // tiles, keys // 128, 32))
+
+
+def moe_route(h, router, top, tiled=None):
     """Per token the `top` experts with the largest softmax scores and their weights: h (T, width),
-    router (E, width) of h's dtype; logits and scores float32. Returns chosen int32 (T, top), in
-    the order of falling score (the lowest index among equals), and weights float32 (T, top) =
-    score / (sum of the chosen scores + 1e-20)."""
+    router (E, width) of h's dtype (`tiled`: its tile-ordered copy, if the caller keeps one). The
+    logits are a product with float32 sums and a float32 result; scores, the choice and the weights
+    are float32. Returns chosen int32 (T, top), in the order of falling score (the lowest index
+    among equals), and weights float32 (T, top) = score / (sum of the chosen scores + 1e-20)."""
     _dev(h, router)
     _need(h.dim() == 2 and router.dim() == 2 and h.shape[1] == router.shape[1] and h.dtype in _DT
           and router.dtype == h.dtype, "h (T, width) and router (E, width) of one dtype")
@@ -480,8 +500,8 @@ def moe_route(h, router, top):
     chosen = torch.empty((T, top), dtype=torch.int32, device=h.device)
     weights = torch.empty((T, top), dtype=torch.float32, device=h.device)
     if T:
-        _check(library("moe").q3_moe_route(_ptr(h), _ptr(router), T, h.shape[1], E, top, _ptr(chosen), _ptr(weights),
-                                           _DT[h.dtype], _stream()), "moe_route")
+        logits = linear(h, router, out_dtype=torch.float32, tiled=tiled)
+        _check(library("moe").q3_moe_pick(_ptr(logits), T, E, top, _ptr(chosen), _ptr(weights), _stream()), "moe_route")
     return chosen, weights
 
 
@@ -506,7 +526,7 @@ def moe_experts(h, chosen, weights, up, down, shared=None, activation="erf"):
         return out
     lib = library("moe")
     P = T * top
-    # bfloat16 with inner sizes in steps of 32: the matrix-core kernel over tiles of 32 slots;
+    # bfloat16 with inner sizes in steps of 32: the matrix-core kernel over tiles of 64 slots;
     # anything else: float32 multiply-adds over tiles of 16
     cores = h.dtype == torch.bfloat16 and width % 32 == 0 and ff % 32 == 0
     tile_rows = lib.q3_moe_tile_rows(1 if cores else 0)

@@ -91,6 +91,6 @@ class LatentAttention(Part):
         ops.headwise_linear(q[:, :, :dn], self.uk, out=rows[:, :, :rank])
         ops.rotate_heads(q[:, :, dn:], rows[:, :, rank:], inv_freq, factor, batch.positions)
         mixed = ops.latent_attention(rows, latent, rank, cache.block_table, batch.cu_seqlens_q, batch.kv_lens,
-                                     batch.max_q_len, self.scale, window=self.window)
+                                     batch.max_q_len, self.scale, window=self.window, max_kv_len=batch.max_kv_len)
         o = ops.headwise_linear(mixed, self.uv)
         return self.out.forward(o.view(-1, H * self.vdim))

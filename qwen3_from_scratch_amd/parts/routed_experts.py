@@ -46,7 +46,7 @@ class RoutedExperts(Part):
 
     def load(self, fetch):
         act, E = self.precision.act, self.experts
-        self.router = fetch(self._name("router"), act)
+        self.router = LinearWeight(fetch(self._name("router"), act), self.precision)
         self.up = torch.stack([fetch(self._name("e%d.up" % e), act, keep=False) for e in range(E)]).contiguous()
         self.down = torch.stack([fetch(self._name("e%d.down" % e), act, keep=False) for e in range(E)]).contiguous()
         if self.shared_ff:
@@ -54,7 +54,7 @@ class RoutedExperts(Part):
             self.shared_down = LinearWeight(fetch(self._name("shared.down"), act), self.precision)
 
     def forward(self, x, batch=None):
-        chosen, weights = ops.moe_route(x, self.router, self.top)
+        chosen, weights = ops.moe_route(x, self.router.weight, self.top, tiled=self.router.tiled)
         shared = None
         if self.shared_ff:
             shared = self.shared_down.forward(ops.gelu(self.shared_up.forward(x), self.activation))

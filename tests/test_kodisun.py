@@ -430,7 +430,8 @@ def test_latent_attention_kernel(dtype, H, Dk, Dv, page, window, general):
     scale = Dk ** -0.5
     if general and not (dtype == torch.bfloat16 and Dk % 32 == 0 and Dv % 16 == 0):
         pytest.skip("these sizes take the general kernel anyway")
-    a = ops.latent_attention(q, cache, Dv, table, cu, kvl, max(q_lens), scale, window=window, general=general)
+    a = ops.latent_attention(q, cache, Dv, table, cu, kvl, max(q_lens), scale, window=window, general=general,
+                             max_kv_len=max(kv))
     b = torch_ops.latent_attention(q, cache, Dv, table, cu, kvl, max(q_lens), scale, window=window)
     assert a.shape == (sum(q_lens), H, Dv)
     assert float((a.float() - b.float()).abs().max()) <= (2e-5 if dtype == torch.float32 else 3e-2)
@@ -449,6 +450,33 @@ def test_latent_attention_kernel(dtype, H, Dk, Dv, page, window, general):
         want = rows[seq][target, :Dv].float().cuda()
         close = float((got - want[None, :]).abs().max()) <= 0.05
         assert close == visible, (back, visible)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("H,Dk,Dv,window", [(6, 160, 128, 0), (6, 160, 128, 300), (16, 576, 512, 700), (3, 64, 48, 0)])
+def test_latent_attention_of_single_tokens_over_many_keys(H, Dk, Dv, window):
+    """Steps of one token a sequence: the keys go over several blocks whose shares are merged; one
+    sequence is a token long, one ends just behind a tile's edge."""
+    import torch_ops
+    from qwen3_from_scratch_amd import ops
+
+    kv = [1000, 1, 513, 37, 2048]
+    cache, table, rows = _paged(kv, 16, Dk, torch.bfloat16, 5)
+    cu = torch.arange(len(kv) + 1, dtype=torch.int32).cuda()
+    kvl = torch.tensor(kv, dtype=torch.int32).cuda()
+    q = _rand((len(kv), H, Dk), 3, torch.bfloat16, 1.5)
+    a = ops.latent_attention(q, cache, Dv, table, cu, kvl, 1, Dk ** -0.5, window=window, max_kv_len=max(kv))
+    b = torch_ops.latent_attention(q, cache, Dv, table, cu, kvl, 1, Dk ** -0.5, window=window)
+    assert ops._latent_splits(len(kv), len(kv), H, 1, max(kv), window) > 1
+    assert float((a.float() - b.float()).abs().max()) <= 3e-2
+    for back in (0, 31, 32, 500, window - 1, window, 2047):
+        if back < 0:
+            continue
+        peaked = q.clone()
+        peaked[4] = (rows[4][2047 - back] * 8.0).to(torch.bfloat16).cuda()[None, :]
+        got = ops.latent_attention(peaked, cache, Dv, table, cu, kvl, 1, 1.0, window=window, max_kv_len=max(kv))[4].float()
+        close = float((got - rows[4][2047 - back, :Dv].float().cuda()[None, :]).abs().max()) <= 0.05
+        assert close == (window == 0 or back < window), back
 
 
 @pytest.mark.gpu

@@ -253,7 +253,7 @@ def rotate_heads(x, out, inv_freq, rot_factor, positions):
     return out
 
 
-def latent_attention(q, cache, value_dim, block_table, cu_seqlens_q, kv_lens, max_q_len, scale, window=0, general=False):
+def latent_attention(q, cache, value_dim, block_table, cu_seqlens_q, kv_lens, max_q_len, scale, window=0, general=False, max_kv_len=0):
     T, H, Dk = q.shape
     page = cache.shape[1]
     res = torch.zeros((T, H, value_dim), dtype=torch.float32, device=q.device)
@@ -277,7 +277,7 @@ def latent_attention(q, cache, value_dim, block_table, cu_seqlens_q, kv_lens, ma
     return res.to(q.dtype)
 
 
-def moe_route(h, router, top):
+def moe_route(h, router, top, tiled=None):
     s = torch.softmax(h.float() @ router.float().T, dim=-1)
     best, chosen = torch.topk(s, top, dim=-1)
     return chosen.to(torch.int32), best / (best.sum(dim=-1, keepdim=True) + 1e-20)
