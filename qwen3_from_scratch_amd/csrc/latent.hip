@@ -419,26 +419,24 @@ __global__ __launch_bounds__(256) void latent_attn_mma_kernel(const bf16_t* __re
 #pragma unroll
   for (int nb = 0; nb < NV; ++nb) acc[nb] = lat_f32x4_t{0.f, 0.f, 0.f, 0.f};
   float m_run = -INFINITY, l_run = 0.f;
+  // a tile's pieces on their way from the cache into registers: eight threads a key, each takes
+  // every eighth piece of 16 bytes of its key's row, so that a thread looks its key's page up once
+  // a tile and eight neighbours read 128 bytes in a row
   const int chunks_per_key = Dk >> 3;
-  const int chunks = LMA_BN * chunks_per_key;
-  constexpr int NCH = (KS + 1) / 2;                           // 16-byte pieces of a tile per thread
+  constexpr int NCH = (KS * 4 + 7) / 8;                       // pieces per thread
+  const int my_key = threadIdx.x >> 3, my_sub = threadIdx.x & 7;
   uint4 pre[NCH];
-
-  // a tile's pieces on their way from the cache into registers
   auto fetch = [&](int kt0) {
+    const int kj = kt0 + my_key;
+    const bf16_t* src = nullptr;
+    if (kj < k_end) {
+      const int pg = block_table[(size_t)b * bt_stride + kj / page];
+      if (pg >= 0 && pg < num_pages) src = cache + ((size_t)pg * page + kj % page) * Dk;
+    }
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
-      const int c = threadIdx.x + 256 * i;
-      pre[i] = make_uint4(0, 0, 0, 0);
-      if (c < chunks) {
-        const int j = c / chunks_per_key, d0 = (c - j * chunks_per_key) * 8;
-        const int kj = kt0 + j;
-        if (kj < k_end) {
-          const int pg = block_table[(size_t)b * bt_stride + kj / page];
-          if (pg >= 0 && pg < num_pages)
-            pre[i] = *reinterpret_cast<const uint4*>(cache + ((size_t)pg * page + kj % page) * Dk + d0);
-        }
-      }
+      const int part = my_sub + 8 * i;
+      pre[i] = (src && part < chunks_per_key) ? *reinterpret_cast<const uint4*>(src + 8 * part) : make_uint4(0, 0, 0, 0);
     }
   };
 
@@ -447,11 +445,8 @@ __global__ __launch_bounds__(256) void latent_attn_mma_kernel(const bf16_t* __re
     __syncthreads();                                          // the last tile's readers are done
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
-      const int c = threadIdx.x + 256 * i;
-      if (c < chunks) {
-        const int j = c / chunks_per_key, d0 = (c - j * chunks_per_key) * 8;
-        *reinterpret_cast<uint4*>(kt + j * ldk + d0) = pre[i];
-      }
+      const int part = my_sub + 8 * i;
+      if (part < chunks_per_key) *reinterpret_cast<uint4*>(kt + my_key * ldk + 8 * part) = pre[i];
     }
     __syncthreads();
     // the values' copy: lanes side by side take keys side by side, so that they write runs of a transposed row
@@ -499,21 +494,22 @@ __global__ __launch_bounds__(256) void latent_attn_mma_kernel(const bf16_t* __re
     if (m_new > -INFINITY) {
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
-        const float e = exp2f(fmaf(v[j], scale_log2, -m_new));
+        const float e = __builtin_amdgcn_exp2f(fmaf(v[j], scale_log2, -m_new));   // 2^x; results below the normal range are zero
         sum += e;
         p.e[j] = (__bf16)e;
       }
-      alpha = exp2f(m_run - m_new);
+      alpha = __builtin_amdgcn_exp2f(m_run - m_new);
     } else {
       p.u = make_uint4(0, 0, 0, 0);
     }
     sum = quad_rows_sum(sum);
     l_run = l_run * alpha + sum;
+    const bool moved = __builtin_amdgcn_ballot_w64(m_new != m_run) != 0;      // some row's maximum moved
     m_run = m_new;
 #pragma unroll
     for (int nb = 0; nb < NV; ++nb) {
       if (nb < nv) {
-        acc[nb] *= alpha;
+        if (moved) acc[nb] *= alpha;
         const bf16_t* vr = vt + (16 * nb + col) * LMA_VLD + 4 * grp;
         LatPack a;
         a.h[0] = *reinterpret_cast<const uint2*>(vr);

@@ -231,21 +231,33 @@ __global__ __launch_bounds__(256) void moe_linear_mma_kernel(
 #pragma unroll
     for (int ns = 0; ns < NS; ++ns) acc[mt][ns] = moe_f32x4_t{0.f, 0.f, 0.f, 0.f};
   const int row_blocks = (rows + 15) >> 4;          // the same for every lane
-#pragma unroll 2
-  for (int k0 = 0; k0 < K; k0 += 32) {
-    MoePack a[NS], b[MMA_MT];
+  // U steps of 32 k are asked for together before their matrix instructions run. One slab a
+  // wavefront is the case of few rows, where the weights stream from memory and what counts is
+  // how many loads are on their way.
+  constexpr int U = NS == 1 ? 4 : 2;
+  for (int k0 = 0; k0 < K; k0 += 32 * U) {
+    MoePack a[U][NS], b[U][MMA_MT];
 #pragma unroll
-    for (int ns = 0; ns < NS; ++ns)
-      a[ns].u = wr[ns] ? *reinterpret_cast<const uint4*>(wr[ns] + k0) : make_uint4(0, 0, 0, 0);
+    for (int u = 0; u < U; ++u) {
+      const int k = k0 + 32 * u;
+      const bool in = k < K;
 #pragma unroll
-    for (int mt = 0; mt < MMA_MT; ++mt)
-      b[mt].u = (mt < row_blocks && xr[mt]) ? *reinterpret_cast<const uint4*>(xr[mt] + k0) : make_uint4(0, 0, 0, 0);
+      for (int ns = 0; ns < NS; ++ns)
+        a[u][ns].u = (in && wr[ns]) ? *reinterpret_cast<const uint4*>(wr[ns] + k) : make_uint4(0, 0, 0, 0);
 #pragma unroll
-    for (int mt = 0; mt < MMA_MT; ++mt) {
-      if (mt < row_blocks) {
+      for (int mt = 0; mt < MMA_MT; ++mt)
+        b[u][mt].u = (in && mt < row_blocks && xr[mt]) ? *reinterpret_cast<const uint4*>(xr[mt] + k)
+                                                       : make_uint4(0, 0, 0, 0);
+    }
 #pragma unroll
-        for (int ns = 0; ns < NS; ++ns)
-          acc[mt][ns] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[ns].v, b[mt].v, acc[mt][ns], 0, 0, 0);
+    for (int u = 0; u < U; ++u) {
+#pragma unroll
+      for (int mt = 0; mt < MMA_MT; ++mt) {
+        if (mt < row_blocks) {
+#pragma unroll
+          for (int ns = 0; ns < NS; ++ns)
+            acc[mt][ns] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[u][ns].v, b[u][mt].v, acc[mt][ns], 0, 0, 0);
+        }
       }
     }
   }
@@ -268,22 +280,159 @@ __global__ __launch_bounds__(256) void moe_linear_mma_kernel(
   }
 }
 
+// ---------------------------------------------------------------------------
+// The product for experts with many rows (prompts): tiles of 128 slots by 128 columns, x and W
+// through shared memory in slices of 64 k, two stages (the next slice is read from memory while
+// the current one is multiplied, and written to the other stage behind one barrier a slice). The
+// four wavefronts own 64 x 64 each: per half slice four operands of x and four of W from shared
+// memory (16 bytes a lane; rows padded by 16 bytes, which spreads a read over all banks) for
+// sixteen matrix instructions. Every sum is formed in the same order as in the kernel above.
+// ---------------------------------------------------------------------------
+#define BIG_TM 128
+#define BIG_BN 128
+#define BIG_BK 64
+#define BIG_LD 72   // halfwords per row of a slice: 64 and 8 of padding
+
+__global__ __launch_bounds__(256) void moe_linear_big_kernel(
+    const bf16_t* __restrict__ x, const int* __restrict__ pair_of_slot, int gather, int pairs_per_row,
+    const bf16_t* __restrict__ w, bf16_t* __restrict__ out, const int* __restrict__ tile_expert,
+    const int* __restrict__ tile_first, const int* __restrict__ offsets, const int* __restrict__ n_tiles, int N, int K,
+    int act) {
+  extern __shared__ __align__(16) unsigned char big_smem[];
+  bf16_t* xs = reinterpret_cast<bf16_t*>(big_smem);              // [2][BIG_TM * BIG_LD]
+  bf16_t* ws = xs + 2 * BIG_TM * BIG_LD;                          // [2][BIG_BN * BIG_LD]
+  const int tile = blockIdx.x;
+  if (tile >= n_tiles[0]) return;
+  const int e = tile_expert[tile];
+  const int first = tile_first[tile];
+  const int rows = min(BIG_TM, offsets[e + 1] - first);
+  const int n0 = blockIdx.y * BIG_BN;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int col = lane & 15, grp = lane >> 4;
+  const int wm = wave >> 1, wn = wave & 1;
+  // what this thread brings in per slice: four pieces of x and four of W (rows r, r + 32, ..., 16 bytes at 8 c)
+  const int r = threadIdx.x >> 3, c = threadIdx.x & 7;
+  const bf16_t* xsrc[4];
+  const bf16_t* wsrc[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int m = r + 32 * i;
+    xsrc[i] = nullptr;
+    if (m < rows) {
+      const int src = gather ? pair_of_slot[first + m] / pairs_per_row : first + m;
+      xsrc[i] = x + (size_t)src * K + 8 * c;
+    }
+    const int n = n0 + r + 32 * i;
+    wsrc[i] = n < N ? w + ((size_t)e * N + n) * K + 8 * c : nullptr;
+  }
+  uint4 px[4], pw[4];
+  auto fetch = [&](int k0) {
+    const bool in = k0 + 8 * c < K;              // K is a multiple of 32: the last slice may be half a slice
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      px[i] = (in && xsrc[i]) ? *reinterpret_cast<const uint4*>(xsrc[i] + k0) : make_uint4(0, 0, 0, 0);
+      pw[i] = (in && wsrc[i]) ? *reinterpret_cast<const uint4*>(wsrc[i] + k0) : make_uint4(0, 0, 0, 0);
+    }
+  };
+  auto stash = [&](int stage) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      *reinterpret_cast<uint4*>(xs + stage * BIG_TM * BIG_LD + (r + 32 * i) * BIG_LD + 8 * c) = px[i];
+      *reinterpret_cast<uint4*>(ws + stage * BIG_BN * BIG_LD + (r + 32 * i) * BIG_LD + 8 * c) = pw[i];
+    }
+  };
+  moe_f32x4_t acc[4][4];
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+    for (int ns = 0; ns < 4; ++ns) acc[mt][ns] = moe_f32x4_t{0.f, 0.f, 0.f, 0.f};
+  const int row_blocks = min(4, max(0, (rows - 64 * wm + 15) >> 4));   // of this wavefront's 64 rows
+  fetch(0);
+  stash(0);
+  __syncthreads();
+  int stage = 0;
+  for (int k0 = 0; k0 < K; k0 += BIG_BK) {
+    const bool more = k0 + BIG_BK < K;
+    if (more) fetch(k0 + BIG_BK);
+    const bf16_t* xt = xs + stage * BIG_TM * BIG_LD;
+    const bf16_t* wt = ws + stage * BIG_BN * BIG_LD;
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      MoePack a[4], b[4];
+#pragma unroll
+      for (int ns = 0; ns < 4; ++ns)
+        a[ns].u = *reinterpret_cast<const uint4*>(wt + (64 * wn + 16 * ns + col) * BIG_LD + 32 * half + 8 * grp);
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt)
+        b[mt].u = *reinterpret_cast<const uint4*>(xt + (64 * wm + 16 * mt + col) * BIG_LD + 32 * half + 8 * grp);
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt) {
+        if (mt < row_blocks) {
+#pragma unroll
+          for (int ns = 0; ns < 4; ++ns)
+            acc[mt][ns] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[ns].v, b[mt].v, acc[mt][ns], 0, 0, 0);
+        }
+      }
+    }
+    if (more) stash(stage ^ 1);
+    __syncthreads();
+    stage ^= 1;
+  }
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt) {
+    const int m = 64 * wm + 16 * mt + col;
+    if (m >= rows) continue;
+#pragma unroll
+    for (int ns = 0; ns < 4; ++ns) {
+      const int n = n0 + 64 * wn + 16 * ns + 4 * grp;
+      bf16_t* o = out + (size_t)(first + m) * N + n;
+      if (n + 3 < N && (N & 3) == 0) {
+        union {
+          uint2 u;
+          bf16_t e[4];
+        } pk;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float v = acc[mt][ns][i];
+          pk.e[i] = float_to_bf16(act >= 0 ? moe_gelu(v, act) : v);
+        }
+        *reinterpret_cast<uint2*>(o) = pk.u;
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          if (n + i < N) {
+            const float v = acc[mt][ns][i];
+            o[i] = float_to_bf16(act >= 0 ? moe_gelu(v, act) : v);
+          }
+        }
+      }
+    }
+  }
+}
+
 // out[t, :] = sum_k weights[t, k] * y[slot_of_pair[t * top + k], :] (+ shared[t, :]), float32 sums in
 // the order k = 0, 1, ..., the shared expert last; rounded once.
 template <typename T>
 __global__ void moe_combine_kernel(const T* __restrict__ y, const int* __restrict__ slot_of_pair,
                                    const float* __restrict__ weights, const T* __restrict__ shared,
                                    T* __restrict__ out, int width, int top) {
+  __shared__ int slots[64];
+  __shared__ float share[64];
   const int t = blockIdx.x;
-  for (int j = threadIdx.x; j < width; j += blockDim.x) {
-    float acc = 0.f;
-    for (int k = 0; k < top; ++k) {
-      const int slot = slot_of_pair[(size_t)t * top + k];
-      acc += weights[(size_t)t * top + k] * to_float(y[(size_t)slot * width + j]);
-    }
-    if (shared) acc += to_float(shared[(size_t)t * width + j]);
-    out[(size_t)t * width + j] = from_float<T>(acc);
+  const int kept = min(top, 64);           // a token's first choices wait in shared memory, so that the rows' loads do not wait for them one by one
+  if ((int)threadIdx.x < kept) {
+    slots[threadIdx.x] = slot_of_pair[(size_t)t * top + threadIdx.x];
+    share[threadIdx.x] = weights[(size_t)t * top + threadIdx.x];
   }
+  __syncthreads();
+  const int j = blockIdx.y * blockDim.x + threadIdx.x;
+  if (j >= width) return;
+  float acc = 0.f;
+  for (int k = 0; k < kept; ++k) acc += share[k] * to_float(y[(size_t)slots[k] * width + j]);
+  for (int k = kept; k < top; ++k)
+    acc += weights[(size_t)t * top + k] * to_float(y[(size_t)slot_of_pair[(size_t)t * top + k] * width + j]);
+  if (shared) acc += to_float(shared[(size_t)t * width + j]);
+  out[(size_t)t * width + j] = from_float<T>(acc);
 }
 
 extern "C" int q3_moe_pick(const float* logits, int n_tokens, int E, int top, int* chosen, float* weights,
@@ -296,12 +445,14 @@ extern "C" int q3_moe_pick(const float* logits, int n_tokens, int E, int top, in
   return q3_launch_status();
 }
 
-// Slots per tile: 16 for the float32 multiply-add kernel, 64 for the matrix-core kernel.
-extern "C" int q3_moe_tile_rows(int matrix_cores) { return matrix_cores ? MMA_TM : MOE_BM; }
+// Slots per tile: 16 for the float32 multiply-add kernel, 64 for the matrix-core kernel, 128 for
+// its form for experts with many rows (`matrix_cores` 0, 1, 2).
+extern "C" int q3_moe_tile_rows(int matrix_cores) { return matrix_cores == 2 ? BIG_TM : matrix_cores ? MMA_TM : MOE_BM; }
 
 extern "C" int q3_moe_align(const int* chosen, int P, int E, int tile_rows, int* offsets, int* pair_of_slot,
                             int* slot_of_pair, int* tile_expert, int* tile_first, int* n_tiles, hipStream_t stream) {
-  if (P <= 0 || E <= 0 || E > 4096 || (tile_rows != MOE_BM && tile_rows != MMA_TM)) return Q3_ERR_BAD_ARGUMENT;
+  if (P <= 0 || E <= 0 || E > 4096 || (tile_rows != MOE_BM && tile_rows != MMA_TM && tile_rows != BIG_TM))
+    return Q3_ERR_BAD_ARGUMENT;
   hipLaunchKernelGGL(moe_align_kernel, dim3(1), dim3(1024), (size_t)2 * E * sizeof(int), stream, chosen, P, E,
                      tile_rows, offsets, pair_of_slot, slot_of_pair, tile_expert, tile_first, n_tiles);
   return q3_launch_status();
@@ -310,9 +461,22 @@ extern "C" int q3_moe_align(const int* chosen, int P, int E, int tile_rows, int*
 // The matrix-core product: bfloat16, K a multiple of 32, tiles of 64 slots.
 extern "C" int q3_moe_linear_mma(const void* x, const int* pair_of_slot, int gather, int pairs_per_row, const void* w,
                                  void* out, const int* tile_expert, const int* tile_first, const int* offsets,
-                                 const int* n_tiles, int max_tiles, int N, int K, int act, hipStream_t stream) {
-  if (max_tiles <= 0 || N <= 0 || K <= 0 || K % 32 || pairs_per_row <= 0 || act < -1 || act > 1)
+                                 const int* n_tiles, int max_tiles, int N, int K, int act, int tile_rows,
+                                 hipStream_t stream) {
+  if (max_tiles <= 0 || N <= 0 || K <= 0 || K % 32 || pairs_per_row <= 0 || act < -1 || act > 1 ||
+      (tile_rows != MMA_TM && tile_rows != BIG_TM))
     return Q3_ERR_BAD_ARGUMENT;
+  if (tile_rows == BIG_TM) {
+    const dim3 big(max_tiles, (N + BIG_BN - 1) / BIG_BN);
+    if (big.y > 65535) return Q3_ERR_UNSUPPORTED;
+    const size_t smem = (size_t)2 * (BIG_TM + BIG_BN) * BIG_LD * sizeof(bf16_t);
+    hipError_t attr = hipFuncSetAttribute((const void*)moe_linear_big_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                          (int)smem);
+    if (attr != hipSuccess) return (int)attr;
+    hipLaunchKernelGGL(moe_linear_big_kernel, big, dim3(256), smem, stream, (const bf16_t*)x, pair_of_slot, gather,
+                       pairs_per_row, (const bf16_t*)w, (bf16_t*)out, tile_expert, tile_first, offsets, n_tiles, N, K, act);
+    return q3_launch_status();
+  }
   // few blocks (steps of few tokens): one slab of 16 columns per wavefront, so that more blocks stream the weights
   const bool narrow = (long)max_tiles * ((N + 255) / 256) < 512;
   const int per_block = narrow ? 64 : 256;
@@ -346,8 +510,10 @@ extern "C" int q3_moe_combine(const void* y, const int* slot_of_pair, const floa
   if (n_tokens <= 0 || width <= 0 || top <= 0) return Q3_ERR_BAD_ARGUMENT;
   int threads = 64;
   while (threads < 256 && threads < width) threads *= 2;
+  if ((width + threads - 1) / threads > 65535) return Q3_ERR_UNSUPPORTED;
   Q3_DISPATCH_DTYPE(dtype, TT,
-                    hipLaunchKernelGGL(moe_combine_kernel<TT>, dim3(n_tokens), dim3(threads), 0, stream, (const TT*)y,
+                    hipLaunchKernelGGL(moe_combine_kernel<TT>, dim3(n_tokens, (width + threads - 1) / threads),
+                                       dim3(threads), 0, stream, (const TT*)y,
                                        slot_of_pair, weights, (const TT*)shared, (TT*)out, width, top));
   return q3_launch_status();
 }

@@ -529,7 +529,8 @@ def moe_experts(h, chosen, weights, up, down, shared=None, activation="erf"):
     # bfloat16 with inner sizes in steps of 32: the matrix-core kernel over tiles of 64 slots;
     # anything else: float32 multiply-adds over tiles of 16
     cores = h.dtype == torch.bfloat16 and width % 32 == 0 and ff % 32 == 0
-    tile_rows = lib.q3_moe_tile_rows(1 if cores else 0)
+    # experts with a hundred rows or more each (prompts): tiles of 128 through shared memory
+    tile_rows = lib.q3_moe_tile_rows((2 if P >= 96 * E else 1) if cores else 0)
     max_tiles = -(-P // tile_rows) + E
     book = torch.empty((E + 1 + 2 * P + 2 * max_tiles + 1,), dtype=torch.int32, device=h.device)
     offsets, pair_of_slot, slot_of_pair = book[:E + 1], book[E + 1:E + 1 + P], book[E + 1 + P:E + 1 + 2 * P]
@@ -543,9 +544,9 @@ def moe_experts(h, chosen, weights, up, down, shared=None, activation="erf"):
     tiles = (_ptr(tile_expert), _ptr(tile_first), _ptr(offsets), _ptr(n_tiles), max_tiles)
     if cores:
         _check(lib.q3_moe_linear_mma(_ptr(h), _ptr(pair_of_slot), 1, top, _ptr(up), _ptr(hidden), *tiles, ff, width,
-                                     GELU_KINDS[activation], stream), "moe_linear")
+                                     GELU_KINDS[activation], tile_rows, stream), "moe_linear")
         _check(lib.q3_moe_linear_mma(_ptr(hidden), _ptr(pair_of_slot), 0, 1, _ptr(down), _ptr(y), *tiles, width, ff,
-                                     -1, stream), "moe_linear")
+                                     -1, tile_rows, stream), "moe_linear")
     else:
         _check(lib.q3_moe_linear(_ptr(h), _ptr(pair_of_slot), 1, top, _ptr(up), _ptr(hidden), *tiles, ff, width,
                                  GELU_KINDS[activation], _DT[h.dtype], stream), "moe_linear")
