@@ -462,20 +462,30 @@ __global__ __launch_bounds__(256) void latent_attn_mma_kernel(const bf16_t* __re
     if (kt0 + LMA_BN < k_end) fetch(kt0 + LMA_BN);            // the next tile travels while this one is worked on
     __syncthreads();
     if (!wave_active || kt0 >= wave_k_end || kt0 + LMA_BN <= wave_k_begin) continue;
-    lat_f32x4_t sc[2];
+    // the two halves of the tile are two chains of matrix instructions that take turns, and the
+    // operands of three steps are asked for together, so that neither a read nor a result is waited for alone
+    lat_f32x4_t sc[2] = {lat_f32x4_t{0.f, 0.f, 0.f, 0.f}, lat_f32x4_t{0.f, 0.f, 0.f, 0.f}};
+    {
+      const bf16_t* kr0 = kt + col * ldk + 8 * grp;
+      const bf16_t* kr1 = kr0 + 16 * ldk;
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
-      lat_f32x4_t c = lat_f32x4_t{0.f, 0.f, 0.f, 0.f};
-      const bf16_t* kr = kt + (16 * kb + col) * ldk + 8 * grp;
+      for (int i0 = 0; i0 < KS; i0 += 3) {
+        LatPack a0[3], a1[3];
 #pragma unroll
-      for (int i = 0; i < KS; ++i) {
-        if (i < ks) {
-          LatPack a;
-          a.u = *reinterpret_cast<const uint4*>(kr + 32 * i);
-          c = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, qreg[i].v, c, 0, 0, 0);
+        for (int u = 0; u < 3; ++u) {
+          if (i0 + u < KS && i0 + u < ks) {
+            a0[u].u = *reinterpret_cast<const uint4*>(kr0 + 32 * (i0 + u));
+            a1[u].u = *reinterpret_cast<const uint4*>(kr1 + 32 * (i0 + u));
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < 3; ++u) {
+          if (i0 + u < KS && i0 + u < ks) {
+            sc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0[u].v, qreg[i0 + u].v, sc[0], 0, 0, 0);
+            sc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1[u].v, qreg[i0 + u].v, sc[1], 0, 0, 0);
+          }
         }
       }
-      sc[kb] = c;
     }
     float v[8];
 #pragma unroll

@@ -284,9 +284,9 @@ __global__ __launch_bounds__(256) void moe_linear_mma_kernel(
 // The product for experts with many rows (prompts): tiles of 128 slots by 128 columns, x and W
 // through shared memory in slices of 64 k, two stages (the next slice is read from memory while
 // the current one is multiplied, and written to the other stage behind one barrier a slice). The
-// four wavefronts own 64 x 64 each: per half slice four operands of x and four of W from shared
-// memory (16 bytes a lane; rows padded by 16 bytes, which spreads a read over all banks) for
-// sixteen matrix instructions. Every sum is formed in the same order as in the kernel above.
+// four wavefronts own 128 x 32 each: per half slice up to eight operands of x and two of W from
+// shared memory (16 bytes a lane; rows padded by 16 bytes, which spreads a read over all banks)
+// for up to sixteen matrix instructions. Every sum is formed in the same order as in the kernel above.
 // ---------------------------------------------------------------------------
 #define BIG_TM 128
 #define BIG_BN 128
@@ -309,7 +309,6 @@ __global__ __launch_bounds__(256) void moe_linear_big_kernel(
   const int n0 = blockIdx.y * BIG_BN;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int col = lane & 15, grp = lane >> 4;
-  const int wm = wave >> 1, wn = wave & 1;
   // what this thread brings in per slice: four pieces of x and four of W (rows r, r + 32, ..., 16 bytes at 8 c)
   const int r = threadIdx.x >> 3, c = threadIdx.x & 7;
   const bf16_t* xsrc[4];
@@ -341,12 +340,14 @@ __global__ __launch_bounds__(256) void moe_linear_big_kernel(
       *reinterpret_cast<uint4*>(ws + stage * BIG_BN * BIG_LD + (r + 32 * i) * BIG_LD + 8 * c) = pw[i];
     }
   };
-  moe_f32x4_t acc[4][4];
+  // a wavefront owns all 128 rows and 32 of the columns: a tile with fewer rows then costs every
+  // wavefront less (an expert's last tile holds what is left of its rows), none of them idles
+  moe_f32x4_t acc[8][2];
 #pragma unroll
-  for (int mt = 0; mt < 4; ++mt)
+  for (int mt = 0; mt < 8; ++mt)
 #pragma unroll
-    for (int ns = 0; ns < 4; ++ns) acc[mt][ns] = moe_f32x4_t{0.f, 0.f, 0.f, 0.f};
-  const int row_blocks = min(4, max(0, (rows - 64 * wm + 15) >> 4));   // of this wavefront's 64 rows
+    for (int ns = 0; ns < 2; ++ns) acc[mt][ns] = moe_f32x4_t{0.f, 0.f, 0.f, 0.f};
+  const int row_blocks = (rows + 15) >> 4;
   fetch(0);
   stash(0);
   __syncthreads();
@@ -358,18 +359,18 @@ __global__ __launch_bounds__(256) void moe_linear_big_kernel(
     const bf16_t* wt = ws + stage * BIG_BN * BIG_LD;
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
-      MoePack a[4], b[4];
+      MoePack a[2], b[8];
 #pragma unroll
-      for (int ns = 0; ns < 4; ++ns)
-        a[ns].u = *reinterpret_cast<const uint4*>(wt + (64 * wn + 16 * ns + col) * BIG_LD + 32 * half + 8 * grp);
+      for (int ns = 0; ns < 2; ++ns)
+        a[ns].u = *reinterpret_cast<const uint4*>(wt + (32 * wave + 16 * ns + col) * BIG_LD + 32 * half + 8 * grp);
 #pragma unroll
-      for (int mt = 0; mt < 4; ++mt)
-        b[mt].u = *reinterpret_cast<const uint4*>(xt + (64 * wm + 16 * mt + col) * BIG_LD + 32 * half + 8 * grp);
+      for (int mt = 0; mt < 8; ++mt)
+        if (mt < row_blocks) b[mt].u = *reinterpret_cast<const uint4*>(xt + (16 * mt + col) * BIG_LD + 32 * half + 8 * grp);
 #pragma unroll
-      for (int mt = 0; mt < 4; ++mt) {
+      for (int mt = 0; mt < 8; ++mt) {
         if (mt < row_blocks) {
 #pragma unroll
-          for (int ns = 0; ns < 4; ++ns)
+          for (int ns = 0; ns < 2; ++ns)
             acc[mt][ns] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[ns].v, b[mt].v, acc[mt][ns], 0, 0, 0);
         }
       }
@@ -379,12 +380,12 @@ __global__ __launch_bounds__(256) void moe_linear_big_kernel(
     stage ^= 1;
   }
 #pragma unroll
-  for (int mt = 0; mt < 4; ++mt) {
-    const int m = 64 * wm + 16 * mt + col;
+  for (int mt = 0; mt < 8; ++mt) {
+    const int m = 16 * mt + col;
     if (m >= rows) continue;
 #pragma unroll
-    for (int ns = 0; ns < 4; ++ns) {
-      const int n = n0 + 64 * wn + 16 * ns + 4 * grp;
+    for (int ns = 0; ns < 2; ++ns) {
+      const int n = n0 + 32 * wave + 16 * ns + 4 * grp;
       bf16_t* o = out + (size_t)(first + m) * N + n;
       if (n + 3 < N && (N & 3) == 0) {
         union {
