@@ -333,7 +333,7 @@ __global__ __launch_bounds__(256) void latent_attn_kernel(const T* __restrict__ 
 // Both leave a query row in the lanes l, l + 16, l + 32, l + 48, so a row's statistics, weights and
 // sums stay where they are. After S^T a lane holds the scores of keys 4g..4g+3 of both 16-key
 // halves (g = lane / 16); the second product numbers its summed index so that these are the
-// lane's eight, and reads V^T accordingly. Scores, maxima, sums and the output sums are float32;
+// lane's eight, and the transposed copy keeps a row's keys in that order. Scores, maxima, sums and the output sums are float32;
 // weights are rounded to bfloat16 as the second product's operand.
 // ---------------------------------------------------------------------------
 #define LMA_ROWS 64
@@ -358,12 +358,15 @@ __device__ inline bool lma_find_tile(const int* __restrict__ cu_q, int B, int H,
   return false;
 }
 
-// KS: most steps of 32 over Dk; NV: most slabs of 16 over Dv. With `splits` > 1 (blockIdx.y) a
+// KS: most steps of 32 over Dk; NV: most slabs of 16 over Dv that one wavefront sums; HALVES: 1, or 2
+// for wide values: eight wavefronts a block, of which wavefronts w and w + 4 serve the same sixteen rows
+// (both form the scores) and each sums half of the value's columns, so that a wavefront's registers
+// leave room for two wavefronts a SIMD. With `splits` > 1 (blockIdx.y) a
 // block walks its share of the tiles and leaves float32 sums that are not yet divided, with the
 // row's maximum (in the exponent's units) and sum, in `partial` ((rows, splits, Dv + 2) floats,
 // rows numbered (packed token, head)); `latent_attn_merge_kernel` joins the shares in their order.
-template <int KS, int NV>
-__global__ __launch_bounds__(256) void latent_attn_mma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
+template <int KS, int NV, int HALVES>
+__global__ __launch_bounds__(256 * HALVES) void latent_attn_mma_kernel(const bf16_t* __restrict__ q, bf16_t* __restrict__ out,
                                                               const bf16_t* __restrict__ cache, int num_pages,
                                                               const int* __restrict__ block_table, int bt_stride,
                                                               const int* __restrict__ cu_q,
@@ -381,9 +384,12 @@ __global__ __launch_bounds__(256) void latent_attn_mma_kernel(const bf16_t* __re
   const int ldk = Dk + LMA_KPAD;                              // halfwords per key row
   bf16_t* kt = reinterpret_cast<bf16_t*>(lma_smem);           // [32][ldk]
   bf16_t* vt = kt + LMA_BN * ldk;                             // [Dv][LMA_VLD]
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = (threadIdx.x >> 6) & 3, half = threadIdx.x >> 8;
   const int col = lane & 15, grp = lane >> 4;
-  const int ks = Dk >> 5, nv = Dv >> 4;
+  const int ks = Dk >> 5;
+  const int slabs = Dv >> 4, per_half = (slabs + HALVES - 1) / HALVES;
+  const int nb0 = half * per_half;                            // this wavefront's first slab of the value
+  const int nv = max(0, min(per_half, slabs - nb0));
 
   // the block's span of keys (and of that this block's share), and this wavefront's
   const int block_last = min(m0 + LMA_ROWS, n_rows) - 1;
@@ -402,6 +408,8 @@ __global__ __launch_bounds__(256) void latent_attn_mma_kernel(const bf16_t* __re
   const int wave_last = min(w0 + 16, n_rows) - 1;
   const int wave_k_end = wave_active ? base_pos + wave_last / H + 1 : 0;
   const int wave_k_begin = (wave_active && window > 0) ? max(0, base_pos + w0 / H - window + 1) : 0;
+  const bool wave_full = wave_active && w0 + 16 <= n_rows;    // all sixteen rows are rows of the sequence
+  const int wave_first_pos = base_pos + w0 / H, wave_last_pos = base_pos + wave_last / H;
 
   const int R = w0 + col;
   const bool valid = R < n_rows;
@@ -423,43 +431,59 @@ __global__ __launch_bounds__(256) void latent_attn_mma_kernel(const bf16_t* __re
   // every eighth piece of 16 bytes of its key's row, so that a thread looks its key's page up once
   // a tile and eight neighbours read 128 bytes in a row
   const int chunks_per_key = Dk >> 3;
-  constexpr int NCH = (KS * 4 + 7) / 8;                       // pieces per thread
-  const int my_key = threadIdx.x >> 3, my_sub = threadIdx.x & 7;
+  constexpr int PER_KEY = 8 * HALVES;                         // threads a key
+  constexpr int NCH = (KS * 4 + PER_KEY - 1) / PER_KEY;       // pieces per thread
+  const int my_key = threadIdx.x / PER_KEY, my_sub = threadIdx.x % PER_KEY;
   uint4 pre[NCH];
-  auto fetch = [&](int kt0) {
+  // The page of a key is looked up a tile before its row is asked for, so that a tile's loads do
+  // not wait for their addresses: the row's load is one trip to memory, not two in a row.
+  auto lookup = [&](int kt0) -> int {
     const int kj = kt0 + my_key;
-    const bf16_t* src = nullptr;
-    if (kj < k_end) {
-      const int pg = block_table[(size_t)b * bt_stride + kj / page];
-      if (pg >= 0 && pg < num_pages) src = cache + ((size_t)pg * page + kj % page) * Dk;
-    }
+    return kj < k_end ? block_table[(size_t)b * bt_stride + kj / page] : -1;
+  };
+  auto fetch = [&](int kt0, int pg) {
+    const int kj = kt0 + my_key;
+    const bf16_t* src = (pg >= 0 && pg < num_pages) ? cache + ((size_t)pg * page + kj % page) * Dk : nullptr;
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
-      const int part = my_sub + 8 * i;
+      const int part = my_sub + PER_KEY * i;
       pre[i] = (src && part < chunks_per_key) ? *reinterpret_cast<const uint4*>(src + 8 * part) : make_uint4(0, 0, 0, 0);
     }
   };
 
-  if (k_begin < k_end) fetch(k_begin);
+  int next_page = -1;
+  if (k_begin < k_end) {
+    fetch(k_begin, lookup(k_begin));
+    next_page = lookup(k_begin + LMA_BN);
+  }
   for (int kt0 = k_begin; kt0 < k_end; kt0 += LMA_BN) {
     __syncthreads();                                          // the last tile's readers are done
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
-      const int part = my_sub + 8 * i;
+      const int part = my_sub + PER_KEY * i;
       if (part < chunks_per_key) *reinterpret_cast<uint4*>(kt + my_key * ldk + 8 * part) = pre[i];
     }
     __syncthreads();
-    // the values' copy: lanes side by side take keys side by side, so that they write runs of a transposed row
-    for (int item = threadIdx.x; item < LMA_BN * (Dv >> 3); item += 256) {
-      const int j = item & (LMA_BN - 1), d0 = (item >> 5) * 8;
-      LatPack v;
-      v.u = *reinterpret_cast<const uint4*>(kt + j * ldk + d0);
-      unsigned short* dst = reinterpret_cast<unsigned short*>(vt) + d0 * LMA_VLD + j;
-      const unsigned short* e = reinterpret_cast<const unsigned short*>(&v.u);
+    // the values' copy, transposed: a thread takes two neighbouring keys and eight columns, and
+    // writes eight pairs. Within a transposed row the keys stand in the order in which the second
+    // product sums them: key 16 hi + 4 g + lo at place 8 g + 4 hi + lo, so that a lane's eight are
+    // 16 bytes in a row. Lanes side by side take key pairs side by side.
+    for (int item = threadIdx.x; item < (LMA_BN / 2) * (Dv >> 3); item += 256 * HALVES) {
+      const int j = (item & 15) * 2, d0 = (item >> 4) * 8;
+      LatPack v0, v1;
+      v0.u = *reinterpret_cast<const uint4*>(kt + j * ldk + d0);
+      v1.u = *reinterpret_cast<const uint4*>(kt + (j + 1) * ldk + d0);
+      const int place = 8 * ((j >> 2) & 3) + 4 * (j >> 4) + (j & 3);
+      unsigned* dst = reinterpret_cast<unsigned*>(reinterpret_cast<unsigned short*>(vt) + d0 * LMA_VLD + place);
+      const unsigned short* e0 = reinterpret_cast<const unsigned short*>(&v0.u);
+      const unsigned short* e1 = reinterpret_cast<const unsigned short*>(&v1.u);
 #pragma unroll
-      for (int i = 0; i < 8; ++i) dst[i * LMA_VLD] = e[i];
+      for (int i = 0; i < 8; ++i) dst[i * (LMA_VLD / 2)] = (unsigned)e0[i] | ((unsigned)e1[i] << 16);
     }
-    if (kt0 + LMA_BN < k_end) fetch(kt0 + LMA_BN);            // the next tile travels while this one is worked on
+    if (kt0 + LMA_BN < k_end) {                               // the next tile travels while this one is worked on
+      fetch(kt0 + LMA_BN, next_page);
+      next_page = lookup(kt0 + 2 * LMA_BN);
+    }
     __syncthreads();
     if (!wave_active || kt0 >= wave_k_end || kt0 + LMA_BN <= wave_k_begin) continue;
     // the two halves of the tile are two chains of matrix instructions that take turns, and the
@@ -488,42 +512,54 @@ __global__ __launch_bounds__(256) void latent_attn_mma_kernel(const bf16_t* __re
       }
     }
     float v[8];
+    // a tile that every row of the wavefront sees whole needs no masks
+    const bool whole = wave_full && kt0 + LMA_BN <= k_end && kt0 + LMA_BN - 1 <= wave_first_pos &&
+                       (window <= 0 || wave_last_pos - kt0 < window);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int key = kt0 + 16 * (j >> 2) + 4 * grp + (j & 3);
-      bool seen = valid && key <= pos && key < k_end;
-      if (window > 0 && pos - key >= window) seen = false;
-      v[j] = seen ? sc[j >> 2][j & 3] : -INFINITY;
+    for (int j = 0; j < 8; ++j) v[j] = sc[j >> 2][j & 3];
+    if (!whole) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int key = kt0 + 16 * (j >> 2) + 4 * grp + (j & 3);
+        bool seen = valid && key <= pos && key < k_end;
+        if (window > 0 && pos - key >= window) seen = false;
+        if (!seen) v[j] = -INFINITY;
+      }
     }
     float mx = fmaxf(fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3])), fmaxf(fmaxf(v[4], v[5]), fmaxf(v[6], v[7])));
     mx = quad_rows_max(mx);
-    const float m_new = fmaxf(m_run, mx * scale_log2);
+    // The exponent's reference m_run follows the row's maximum only when that has grown by more
+    // than 8 (a factor of 256) since it was set: weights then stay below 256, which float32 sums and
+    // bfloat16 weights carry as well as numbers below 1, and the sums are rescaled a few times a row
+    // instead of once a tile. The result is the same quotient.
+    const float m_tile = mx * scale_log2;
+    const bool rescale = m_tile > m_run + 8.f;                // also the first tile in which the row sees a key
+    float alpha = 1.f;
+    if (rescale) {
+      alpha = __builtin_amdgcn_exp2f(m_run - m_tile);         // 0 from minus infinity
+      m_run = m_tile;
+    }
     LatPack p;
     float sum = 0.f;
-    float alpha = 1.f;
-    if (m_new > -INFINITY) {
+    if (m_run > -INFINITY) {
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
-        const float e = __builtin_amdgcn_exp2f(fmaf(v[j], scale_log2, -m_new));   // 2^x; results below the normal range are zero
+        const float e = __builtin_amdgcn_exp2f(fmaf(v[j], scale_log2, -m_run));   // 2^x; results below the normal range are zero
         sum += e;
         p.e[j] = (__bf16)e;
       }
-      alpha = __builtin_amdgcn_exp2f(m_run - m_new);
     } else {
       p.u = make_uint4(0, 0, 0, 0);
     }
     sum = quad_rows_sum(sum);
     l_run = l_run * alpha + sum;
-    const bool moved = __builtin_amdgcn_ballot_w64(m_new != m_run) != 0;      // some row's maximum moved
-    m_run = m_new;
+    const bool moved = __builtin_amdgcn_ballot_w64(rescale) != 0;
 #pragma unroll
     for (int nb = 0; nb < NV; ++nb) {
       if (nb < nv) {
         if (moved) acc[nb] *= alpha;
-        const bf16_t* vr = vt + (16 * nb + col) * LMA_VLD + 4 * grp;
         LatPack a;
-        a.h[0] = *reinterpret_cast<const uint2*>(vr);
-        a.h[1] = *reinterpret_cast<const uint2*>(vr + 16);
+        a.u = *reinterpret_cast<const uint4*>(vt + (16 * (nb0 + nb) + col) * LMA_VLD + 8 * grp);
         acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, p.v, acc[nb], 0, 0, 0);
       }
     }
@@ -531,13 +567,13 @@ __global__ __launch_bounds__(256) void latent_attn_mma_kernel(const bf16_t* __re
   if (!valid) return;
   if (splits > 1) {
     float* dst = partial + (((size_t)(q0 + tok) * H + head) * splits + blockIdx.y) * (Dv + 2);
-    if (grp == 0) {
+    if (grp == 0 && half == 0) {
       dst[Dv] = m_run;
       dst[Dv + 1] = l_run;
     }
 #pragma unroll
     for (int nb = 0; nb < NV; ++nb) {
-      if (nb < nv) *reinterpret_cast<float4*>(dst + 16 * nb + 4 * grp) = make_float4(acc[nb][0], acc[nb][1], acc[nb][2], acc[nb][3]);
+      if (nb < nv) *reinterpret_cast<float4*>(dst + 16 * (nb0 + nb) + 4 * grp) = make_float4(acc[nb][0], acc[nb][1], acc[nb][2], acc[nb][3]);
     }
     return;
   }
@@ -552,7 +588,7 @@ __global__ __launch_bounds__(256) void latent_attn_mma_kernel(const bf16_t* __re
       } pk;
 #pragma unroll
       for (int i = 0; i < 4; ++i) pk.e[i] = float_to_bf16(acc[nb][i] * inv);
-      *reinterpret_cast<uint2*>(o + 16 * nb) = pk.u;
+      *reinterpret_cast<uint2*>(o + 16 * (nb0 + nb)) = pk.u;
     }
   }
 }
@@ -669,17 +705,17 @@ static int launch_latent_attn(const void* q, void* out, const void* cache, int n
   return q3_launch_status();
 }
 
-template <int KS, int NV>
+template <int KS, int NV, int HALVES>
 static int launch_latent_attn_mma(const void* q, void* out, const void* cache, int num_pages, const int* block_table,
                                   int bt_stride, const int* cu_q, const int* kv_lens, int B, int T, int H, int Dk,
                                   int Dv, int page, float scale, int window, int splits, float* partial,
                                   hipStream_t stream) {
   const size_t smem = (size_t)(LMA_BN * (Dk + LMA_KPAD) + Dv * LMA_VLD) * sizeof(bf16_t);
-  int e = raise_shared_memory((const void*)latent_attn_mma_kernel<KS, NV>, smem);
+  int e = raise_shared_memory((const void*)latent_attn_mma_kernel<KS, NV, HALVES>, smem);
   if (e) return e;
   const long tiles = ((long)T * H) / LMA_ROWS + B;            // at least the sequences' tiles of 64 rows together
   if (tiles > 0x7fffffffL || splits < 1 || splits > 65535 || (splits > 1 && !partial)) return Q3_ERR_UNSUPPORTED;
-  hipLaunchKernelGGL((latent_attn_mma_kernel<KS, NV>), dim3((unsigned)tiles, splits), dim3(256), smem, stream,
+  hipLaunchKernelGGL((latent_attn_mma_kernel<KS, NV, HALVES>), dim3((unsigned)tiles, splits), dim3(256 * HALVES), smem, stream,
                      (const bf16_t*)q, (bf16_t*)out, (const bf16_t*)cache, num_pages, block_table, bt_stride, cu_q,
                      kv_lens, B, H, Dk, Dv, page, scale * 1.44269504088896341f, window, splits, partial);
   if (splits > 1)
@@ -702,12 +738,12 @@ extern "C" int q3_latent_attention(const void* q, void* out, const void* cache, 
   if (Dv > 1024) return Q3_ERR_UNSUPPORTED;
   if (!general && q3_latent_attention_fast_path(Dk, Dv, dtype)) {
     if (Dk <= 192 && Dv <= 128)
-      return launch_latent_attn_mma<6, 8>(q, out, cache, num_pages, block_table, bt_stride, cu_q, kv_lens, B, T, H, Dk,
+      return launch_latent_attn_mma<6, 8, 1>(q, out, cache, num_pages, block_table, bt_stride, cu_q, kv_lens, B, T, H, Dk,
                                           Dv, page, scale, window, splits, partial, stream);
     if (Dk <= 320 && Dv <= 256)
-      return launch_latent_attn_mma<10, 16>(q, out, cache, num_pages, block_table, bt_stride, cu_q, kv_lens, B, T, H,
+      return launch_latent_attn_mma<10, 16, 1>(q, out, cache, num_pages, block_table, bt_stride, cu_q, kv_lens, B, T, H,
                                             Dk, Dv, page, scale, window, splits, partial, stream);
-    return launch_latent_attn_mma<18, 32>(q, out, cache, num_pages, block_table, bt_stride, cu_q, kv_lens, B, T, H, Dk,
+    return launch_latent_attn_mma<18, 16, 2>(q, out, cache, num_pages, block_table, bt_stride, cu_q, kv_lens, B, T, H, Dk,
                                           Dv, page, scale, window, splits, partial, stream);
   }
   Q3_DISPATCH_DTYPE(dtype, TT, {
