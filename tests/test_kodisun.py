@@ -73,7 +73,16 @@ WIDE = {
         {"type": "latent_attention", "mixer": _mixer(8, 64, 32, 32, 96, 128, 70), "mlp": _mlp(4, 3, 128, 64)},
         {"type": "latent_attention", "mixer": _mixer(4, 32, 64, 64, 32, 64, 0), "mlp": None},
     ]}
-CONFIGS = {"looped": LOOPED, "plain": PLAIN, "wide": WIDE}
+# sizes that no vector access and no matrix instruction takes: everything goes through the general kernels;
+# one head, one expert, a loop of one pass over the only two layers
+ODD = {
+    "architecture": "Kodisun", "vocab": 53, "width": 40, "norm": {"eps": 1e-5},
+    "loop": {"start": 0, "stop": 2, "times": 1},
+    "layers": [
+        {"type": "latent_attention", "mixer": _mixer(3, 10, 6, 14, 12, 20, 5, dims=4), "mlp": _mlp(3, 2, 18, 10)},
+        {"type": "latent_attention", "mixer": _mixer(1, 6, 2, 3, 5, 7, 0), "mlp": _mlp(1, 1, 9, 0)},
+    ]}
+CONFIGS = {"looped": LOOPED, "plain": PLAIN, "wide": WIDE, "odd": ODD}
 
 
 def _write(folder, data, seed=5, std=0.2, peak=None):
