@@ -66,15 +66,26 @@ def load_model_config(model_dir):
         raise ConfigError("no config.json in %s" % model_dir)
     with open(path) as fh:
         data = json.load(fh)
+    return config_from_dict(data)
+
+
+def architecture_named_by(data):
+    """The architecture's name in a config.json's dict: the first of `architectures`, or the one
+    string `architecture` that some architectures name themselves with."""
     names = data.get("architectures")
     if names is None and isinstance(data.get("architecture"), str):
-        names = [data["architecture"]]           # some architectures name themselves with one string
+        names = [data["architecture"]]
     if not names or not isinstance(names, list):
         raise ConfigError(
             "config.json: 'architectures' (or 'architecture') must name the model class; known: %s"
             % ", ".join(architectures())
         )
-    config_class, _ = lookup_architecture(names[0])
+    return names[0]
+
+
+def config_from_dict(data):
+    """A config.json's dict as the typed configuration of the architecture it names."""
+    config_class, _ = lookup_architecture(architecture_named_by(data))
     return config_class.from_dict(data)
 
 

@@ -59,13 +59,12 @@ def main(argv=None):
     if args.write_random:
         if not args.from_config:
             p.error("--write_random needs --from_config")
-        from ..config.registry import lookup_architecture
+        from ..config.registry import config_from_dict
         from ..weights import write_random_model
 
         with open(args.from_config) as fh:
             data = json.load(fh)
-        config_class, _ = lookup_architecture(data["architectures"][0])
-        write_random_model(args.write_random, config_class.from_dict(data), seed=args.seed, std=args.std,
+        write_random_model(args.write_random, config_from_dict(data), seed=args.seed, std=args.std,
                            norm_jitter=args.norm_jitter)
         print("wrote %s" % args.write_random)
         return 0

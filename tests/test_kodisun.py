@@ -607,3 +607,59 @@ def test_replay_program(folders, tmp_path, dtype):
             for key, row in zip(wanted, data):
                 got[key] = torch.from_numpy(row.copy())
     assert _off(got, want, dtype) <= 1.0
+
+
+def test_command_line_writes_a_folder_from_the_nested_config(tmp_path):
+    """`--write_random` reads the architecture's name from the one string this config.json has."""
+    from qwen3_from_scratch_amd.engine.cli import main
+
+    source = tmp_path / "config.json"
+    source.write_text(json.dumps(PLAIN))
+    assert main(["--write_random", str(tmp_path / "m"), "--from_config", str(source), "--seed", "3"]) == 0
+    assert load_model_config(str(tmp_path / "m")).to_dict() == PLAIN
+    names = set(load_file(str(tmp_path / "m" / "model.safetensors")))
+    assert "l1.mlp.e2.down" in names and "loop.step" not in names
+
+
+@pytest.mark.gpu
+def test_command_line_generates(tmp_path):
+    folder = _write(tmp_path / "m", WIDE, peak=3.0)
+    config, w, _ = _truth(folder, {})
+    prompt = random_tokens(50, WIDE["vocab"], 12)
+    proc = subprocess.run(
+        [sys.executable, "-m", "qwen3_from_scratch_amd", "--path", folder, "--dtype", "float32", "--prompt_ids",
+         ",".join(map(str, prompt)), "--max_new_tokens", "6", "--temperature", "0", "--ignore_eos", "--max_len", "128",
+         "--block_size", "16", "--num_blocks", "16", "--max_num_seqs", "2"],
+        capture_output=True, text=True, timeout=600, cwd=ROOT)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    got = [int(t) for t in proc.stdout.split()]
+    seq = list(prompt)
+    for _ in range(6):
+        seq.append(int(torch.argmax(plain.logits_of_sequence(config, w, seq)[-1])))
+    assert got == seq[len(prompt):]
+
+
+def test_requests_share_a_prefix_where_no_layer_has_a_window(cpu_ops, tmp_path):
+    """Without windows the latent rows of a shared beginning are pages like any other's: a second
+    request takes them over, in every pass's plane, and generates what it would have alone."""
+    data = copy.deepcopy(LOOPED)
+    for layer in data["layers"]:
+        layer["mixer"].pop("mask", None)
+    folder = _write(tmp_path / "m", data, peak=3.0)
+    config, w, _ = _truth(folder, {})
+    engine = SyncEngine(path=folder, dtype="float32", device="cpu", max_len=128, block_size=8, num_blocks=40,
+                        max_num_seqs=2, max_num_tokens=32, chunked_prefill_size=16, enable_prefix_cache=True)
+    assert engine.runner.manager.prefix_cache
+    stem = random_tokens(29, data["vocab"], 21)
+    prompts = [stem + random_tokens(5, data["vocab"], 22), stem + random_tokens(9, data["vocab"], 23)]
+    got = [engine.generate_ids([p], max_new_tokens=4, temperature=0.0, ignore_eos=True)[0] for p in prompts]
+    assert engine.runner.manager.prefix_hits == 24            # three blocks of eight
+    for prompt, new in zip(prompts, got):
+        seq = list(prompt)
+        for _ in range(4):
+            seq.append(int(torch.argmax(plain.logits_of_sequence(config, w, seq)[-1])))
+        assert new == seq[len(prompt):]
+    # with a window anywhere the index stays off
+    windowed = SyncEngine(path=_write(tmp_path / "w", LOOPED), dtype="float32", device="cpu", max_len=128, block_size=8,
+                          num_blocks=40, max_num_seqs=2, enable_prefix_cache=True)
+    assert not windowed.runner.manager.prefix_cache
