@@ -61,7 +61,7 @@ LOOPED = {
 PLAIN = {
     "architecture": "Kodisun", "vocab": 97, "width": 64, "norm": {"eps": 1e-6},
     "layers": [
-        {"type": "latent_attention", "mixer": _mixer(2, 32, 32, 48, 24, 64, 1), "mlp": _mlp(8, 3, 32, 48)},
+        {"type": "latent_attention", "mixer": _mixer(2, 32, 32, 48, 24, 64, 1), "mlp": _mlp(7, 3, 32, 48)},
         {"type": "latent_attention", "mixer": _mixer(6, 16, 16, 32, 40, 48, 500, scaling=YARN), "mlp": _mlp(3, 2, 64, 32)},
     ]}
 # sizes in steps that the matrix-core kernels take, the loop from the first layer on
@@ -202,7 +202,7 @@ def test_rotation_frequencies_with_and_without_blending():
     from qwen3_from_scratch_amd.parts.position import RotaryPairs
     from qwen3_from_scratch_amd.parts.base import Precision
 
-    for rot in ({"dims": 12, "base": 500.0}, {"dims": 32, "base": 20000.0, "scaling": YARN},
+    for rot in ({"dims": 12, "base": 500.0}, {"dims": 24, "base": 30000.0, "scaling": YARN},
                 {"dims": 8, "base": 10000.0, "scaling": {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}}):
         scaling = rot.get("scaling")
         part = RotaryPairs("", Precision(torch.float32), "cpu", rot["dims"], rot["base"],
@@ -212,8 +212,8 @@ def test_rotation_frequencies_with_and_without_blending():
         assert torch.allclose(part.frequencies()[0].double(), torch.tensor(freqs, dtype=torch.float64), rtol=1e-7)
         assert abs(part.frequencies()[1] - factor) < 1e-12
     # the blend really changes the slow pairs and leaves the fastest alone
-    blended, factor = plain.rotation_frequencies({"dims": 32, "base": 20000.0, "scaling": YARN})
-    straight, _ = plain.rotation_frequencies({"dims": 32, "base": 20000.0})
+    blended, factor = plain.rotation_frequencies({"dims": 24, "base": 30000.0, "scaling": YARN})
+    straight, _ = plain.rotation_frequencies({"dims": 24, "base": 30000.0})
     assert blended[0] == straight[0] and abs(blended[-1] - straight[-1] / 4.0) < 1e-15 and factor > 1.0
 
 
@@ -329,7 +329,7 @@ def test_gelu_kernel(dtype):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("q_rank,kv_rank,rot_dim,pairs", [(20, 40, 8, 4), (96, 128, 32, 16), (33, 7, 10, 3)])
+@pytest.mark.parametrize("q_rank,kv_rank,rot_dim,pairs", [(20, 40, 8, 4), (80, 144, 24, 12), (33, 7, 10, 3)])
 def test_latent_prepare_kernel(dtype, q_rank, kv_rank, rot_dim, pairs):
     import torch_ops
     from qwen3_from_scratch_amd import ops
@@ -420,7 +420,7 @@ def _paged(rows_per_seq, page, Dk, dtype, seed):
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("general", [False, True])
-@pytest.mark.parametrize("H,Dk,Dv,page,window", [(3, 48, 40, 8, 19), (6, 160, 128, 16, 40), (5, 36, 24, 16, 0),
+@pytest.mark.parametrize("H,Dk,Dv,page,window", [(3, 48, 40, 8, 19), (5, 160, 112, 16, 37), (5, 36, 24, 16, 0),
                                                  (16, 96, 64, 32, 70), (2, 200, 136, 8, 1), (4, 576, 512, 16, 100),
                                                  (8, 288, 256, 16, 0), (7, 64, 16, 8, 33)])
 def test_latent_attention_kernel(dtype, H, Dk, Dv, page, window, general):
@@ -462,7 +462,7 @@ def test_latent_attention_kernel(dtype, H, Dk, Dv, page, window, general):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("H,Dk,Dv,window", [(6, 160, 128, 0), (6, 160, 128, 300), (16, 576, 512, 700), (3, 64, 48, 0)])
+@pytest.mark.parametrize("H,Dk,Dv,window", [(5, 160, 112, 0), (5, 160, 112, 300), (16, 576, 512, 700), (3, 64, 48, 0)])
 def test_latent_attention_of_single_tokens_over_many_keys(H, Dk, Dv, window):
     """Steps of one token a sequence: the keys go over several blocks whose shares are merged; one
     sequence is a token long, one ends just behind a tile's edge."""
@@ -490,7 +490,7 @@ def test_latent_attention_of_single_tokens_over_many_keys(H, Dk, Dv, window):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("T,width,E,top", [(1, 64, 8, 3), (77, 48, 5, 5), (300, 256, 70, 6), (9, 33, 3, 1)])
+@pytest.mark.parametrize("T,width,E,top", [(1, 64, 9, 4), (77, 48, 5, 5), (300, 192, 70, 6), (9, 33, 3, 1)])
 def test_router_kernel(dtype, T, width, E, top):
     h, router = _rand((T, width), 1, dtype), _rand((E, width), 2, dtype, 0.5)
     (chosen, weights), (chosen_t, weights_t) = _both("moe_route", h, router, top)
@@ -507,7 +507,7 @@ def test_router_kernel(dtype, T, width, E, top):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("T,width,ff,E,top,shared", [(1, 64, 32, 8, 3, True), (50, 48, 24, 5, 2, False),
+@pytest.mark.parametrize("T,width,ff,E,top,shared", [(1, 64, 32, 7, 3, True), (50, 48, 24, 5, 2, False),
                                                       (333, 128, 96, 6, 3, True), (17, 40, 20, 4, 4, True),
                                                       (5, 256, 64, 64, 1, False), (700, 96, 160, 3, 2, True),
                                                       (900, 64, 96, 2, 2, False)])
