@@ -2,6 +2,7 @@
 // experts per token, the (token, choice) pairs put in the order of their experts, the experts'
 // products over those runs of rows, and the weighted sum per token.
 #include "common.h"
+#include "gemm_tiles.h"
 
 #include <math.h>
 
@@ -411,6 +412,136 @@ __global__ __launch_bounds__(256) void moe_linear_big_kernel(
   }
 }
 
+// ---------------------------------------------------------------------------
+// The same product with the dense path's machinery (gemm_tiles.h): K a multiple of 64; tiles of
+// 128 sorted rows by 128 columns; slices of 64 k travel from memory into shared memory by loads
+// that write it directly, three slices ahead of the one that is multiplied (four stages), their
+// 16-byte pieces placed by the same XOR, so that operand reads meet no bank conflict; four
+// wavefronts of 64 x 64. What differs from the dense kernel is where a tile's rows come from:
+// the tile's expert gives the weight, its rows of x are gathered by index (a row beyond the
+// tile's count reads the tile's last row and is never written).
+// ---------------------------------------------------------------------------
+#define GT_BM 256
+#define GT_BN 128
+#define GT_WM 4
+#define GT_STAGES 3
+
+__global__ __launch_bounds__(64 * GT_WM * 2) void moe_linear_tiles_kernel(
+    const bf16_t* __restrict__ x, const int* __restrict__ pair_of_slot, int gather, int pairs_per_row,
+    const bf16_t* __restrict__ w, bf16_t* __restrict__ out, const int* __restrict__ tile_expert,
+    const int* __restrict__ tile_first, const int* __restrict__ offsets, const int* __restrict__ n_tiles, int N, int K,
+    int act) {
+  using namespace tiles;
+  typedef Shape<GT_BM, GT_BN, GT_WM, 2, GT_STAGES> S;
+  extern __shared__ __attribute__((aligned(16))) unsigned char gt_smem[];
+  const int tile = blockIdx.x;
+  if (tile >= n_tiles[0]) return;
+  const int e = tile_expert[tile];
+  const int first_row = tile_first[tile];
+  const int rows = min(GT_BM, offsets[e + 1] - first_row);
+  const int n0 = blockIdx.y * GT_BN;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int col = lane & 15, grp = lane >> 4;
+  const int wm = wave % GT_WM, wn = wave / GT_WM;
+  const int piece = (tid & 7) ^ ((tid >> 4) & 7);
+  const bf16_t* x_src[S::X_TURNS];
+  const bf16_t* w_src[S::W_TURNS];
+#pragma unroll
+  for (int j = 0; j < S::X_TURNS; ++j) {
+    const int slot = first_row + min(S::TURN_ROWS * j + (tid >> 3), rows - 1);
+    const int src = gather ? pair_of_slot[slot] / pairs_per_row : slot;
+    x_src[j] = x + (size_t)src * K + 8 * piece;
+  }
+  const bf16_t* we = w + (size_t)e * N * K;
+#pragma unroll
+  for (int j = 0; j < S::W_TURNS; ++j)
+    w_src[j] = we + (size_t)min(n0 + S::TURN_ROWS * j + (tid >> 3), N - 1) * K + 8 * piece;
+  typedef __attribute__((address_space(3))) unsigned char* lds_ptr;
+  const unsigned smem_lds = (unsigned)(unsigned long)(lds_ptr)gt_smem;
+  auto load_to_lds = [&](const void* src, unsigned lds) {
+    asm volatile("s_mov_b32 m0, %1\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(lds) : "memory", "m0");
+  };
+  auto copy_step = [&](int kt, int stage) {
+    const unsigned base = __builtin_amdgcn_readfirstlane(smem_lds + stage * S::STAGE_BYTES + 1024 * wave);
+#pragma unroll
+    for (int j = 0; j < S::X_TURNS; ++j) load_to_lds(x_src[j] + (size_t)kt * BK, base + 16 * S::THREADS * j);
+#pragma unroll
+    for (int j = 0; j < S::W_TURNS; ++j)
+      load_to_lds(w_src[j] + (size_t)kt * BK, base + GT_BM * ROW_BYTES + 16 * S::THREADS * j);
+  };
+  // loads complete in the order they were issued: with no more than the later steps' loads
+  // outstanding, this thread's share of the next step has landed
+  auto wait_for_step = [&](int steps_after) {
+    if (steps_after <= 0)
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    else
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(S::LOADS) : "memory");
+  };
+  static_assert(GT_STAGES == 3 && S::LOADS < 64, "the wait counts above");
+  const int swz = (col >> 1) & 7;
+  int read_off[2];
+#pragma unroll
+  for (int s = 0; s < 2; ++s) read_off[s] = col * ROW_BYTES + 16 * ((4 * s + grp) ^ swz);
+  const int x_half = wm * (GT_BM / GT_WM) * ROW_BYTES, w_half = GT_BM * ROW_BYTES + wn * (GT_BN / 2) * ROW_BYTES;
+  f32x4_t acc[S::MI][S::NJ];
+#pragma unroll
+  for (int i = 0; i < S::MI; ++i)
+#pragma unroll
+    for (int j = 0; j < S::NJ; ++j) acc[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  const int row_blocks = min(S::MI, max(0, (rows - wm * (GT_BM / GT_WM) + 15) >> 4));   // of this wavefront's 64 rows
+  const int steps = K / BK;
+#pragma unroll
+  for (int ahead = 0; ahead < GT_STAGES - 1; ++ahead)
+    if (ahead < steps) copy_step(ahead, ahead);
+  for (int kt = 0; kt < steps; ++kt) {
+    wait_for_step(min(kt + GT_STAGES - 2, steps - 1) - kt);
+    __syncthreads();
+    if (kt + GT_STAGES - 1 < steps) copy_step(kt + GT_STAGES - 1, (kt + GT_STAGES - 1) % GT_STAGES);
+    const unsigned char* st = gt_smem + (kt % GT_STAGES) * S::STAGE_BYTES;
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      Frag xf[S::MI], wf[S::NJ];
+#pragma unroll
+      for (int i = 0; i < S::MI; ++i)
+        xf[i].u = *reinterpret_cast<const uint4*>(st + x_half + 16 * i * ROW_BYTES + read_off[s]);
+#pragma unroll
+      for (int j = 0; j < S::NJ; ++j)
+        wf[j].u = *reinterpret_cast<const uint4*>(st + w_half + 16 * j * ROW_BYTES + read_off[s]);
+#pragma unroll
+      for (int i = 0; i < S::MI; ++i) {
+        if (i < row_blocks) {
+#pragma unroll
+          for (int j = 0; j < S::NJ; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[j].v, xf[i].v, acc[i][j], 0, 0, 0);
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < S::MI; ++i) {
+    const int m = wm * (GT_BM / GT_WM) + 16 * i + col;
+    if (m >= rows) continue;
+#pragma unroll
+    for (int j = 0; j < S::NJ; ++j) {
+      const int n = n0 + wn * (GT_BN / 2) + 16 * j + 4 * grp;
+      if (n >= N) continue;
+      f32x4_t c = acc[i][j];
+      if (act >= 0) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) c[q] = moe_gelu(c[q], act);
+      }
+      bf16_t* o = out + (size_t)(first_row + m) * N + n;
+      if (n + 3 < N && (N % 4) == 0) {
+        *reinterpret_cast<uint2*>(o) = pack_bf16x4(c);
+      } else {
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          if (n + q < N) o[q] = float_to_bf16(c[q]);
+      }
+    }
+  }
+}
+
 // out[t, :] = sum_k weights[t, k] * y[slot_of_pair[t * top + k], :] (+ shared[t, :]), float32 sums in
 // the order k = 0, 1, ..., the shared expert last; rounded once.
 template <typename T>
@@ -447,12 +578,15 @@ extern "C" int q3_moe_pick(const float* logits, int n_tokens, int E, int top, in
 }
 
 // Slots per tile: 16 for the float32 multiply-add kernel, 64 for the matrix-core kernel, 128 for
-// its form for experts with many rows (`matrix_cores` 0, 1, 2).
-extern "C" int q3_moe_tile_rows(int matrix_cores) { return matrix_cores == 2 ? BIG_TM : matrix_cores ? MMA_TM : MOE_BM; }
+// its form for experts with many rows, 256 for that with inner sizes in steps of 64 (`matrix_cores` 0, 1, 2, 3).
+extern "C" int q3_moe_tile_rows(int matrix_cores) {
+  return matrix_cores == 3 ? GT_BM : matrix_cores == 2 ? BIG_TM : matrix_cores ? MMA_TM : MOE_BM;
+}
 
 extern "C" int q3_moe_align(const int* chosen, int P, int E, int tile_rows, int* offsets, int* pair_of_slot,
                             int* slot_of_pair, int* tile_expert, int* tile_first, int* n_tiles, hipStream_t stream) {
-  if (P <= 0 || E <= 0 || E > 4096 || (tile_rows != MOE_BM && tile_rows != MMA_TM && tile_rows != BIG_TM))
+  if (P <= 0 || E <= 0 || E > 4096 ||
+      (tile_rows != MOE_BM && tile_rows != MMA_TM && tile_rows != BIG_TM && tile_rows != GT_BM))
     return Q3_ERR_BAD_ARGUMENT;
   hipLaunchKernelGGL(moe_align_kernel, dim3(1), dim3(1024), (size_t)2 * E * sizeof(int), stream, chosen, P, E,
                      tile_rows, offsets, pair_of_slot, slot_of_pair, tile_expert, tile_first, n_tiles);
@@ -465,8 +599,20 @@ extern "C" int q3_moe_linear_mma(const void* x, const int* pair_of_slot, int gat
                                  const int* n_tiles, int max_tiles, int N, int K, int act, int tile_rows,
                                  hipStream_t stream) {
   if (max_tiles <= 0 || N <= 0 || K <= 0 || K % 32 || pairs_per_row <= 0 || act < -1 || act > 1 ||
-      (tile_rows != MMA_TM && tile_rows != BIG_TM))
+      (tile_rows != MMA_TM && tile_rows != BIG_TM && tile_rows != GT_BM))
     return Q3_ERR_BAD_ARGUMENT;
+  if (tile_rows == GT_BM) {         // the dense path's copies and stages
+    typedef tiles::Shape<GT_BM, GT_BN, GT_WM, 2, GT_STAGES> S;
+    const dim3 grid(max_tiles, (N + GT_BN - 1) / GT_BN);
+    if (grid.y > 65535 || K % 64) return Q3_ERR_UNSUPPORTED;
+    hipError_t attr = hipFuncSetAttribute((const void*)moe_linear_tiles_kernel,
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, S::SMEM_BYTES);
+    if (attr != hipSuccess) return (int)attr;
+    hipLaunchKernelGGL(moe_linear_tiles_kernel, grid, dim3(S::THREADS), S::SMEM_BYTES, stream, (const bf16_t*)x,
+                       pair_of_slot, gather, pairs_per_row, (const bf16_t*)w, (bf16_t*)out, tile_expert, tile_first,
+                       offsets, n_tiles, N, K, act);
+    return q3_launch_status();
+  }
   if (tile_rows == BIG_TM) {
     const dim3 big(max_tiles, (N + BIG_BN - 1) / BIG_BN);
     if (big.y > 65535) return Q3_ERR_UNSUPPORTED;

@@ -530,7 +530,9 @@ def moe_experts(h, chosen, weights, up, down, shared=None, activation="erf"):
     # anything else: float32 multiply-adds over tiles of 16
     cores = h.dtype == torch.bfloat16 and width % 32 == 0 and ff % 32 == 0
     # experts with a hundred rows or more each (prompts): tiles of 128 through shared memory
-    tile_rows = lib.q3_moe_tile_rows((2 if P >= 96 * E else 1) if cores else 0)
+    # (with inner sizes in steps of 64: tiles of 256 by the dense path's copies and stages)
+    many = 3 if width % 64 == 0 and ff % 64 == 0 else 2
+    tile_rows = lib.q3_moe_tile_rows((many if P >= 96 * E else 1) if cores else 0)
     max_tiles = -(-P // tile_rows) + E
     book = torch.empty((E + 1 + 2 * P + 2 * max_tiles + 1,), dtype=torch.int32, device=h.device)
     offsets, pair_of_slot, slot_of_pair = book[:E + 1], book[E + 1:E + 1 + P], book[E + 1 + P:E + 1 + 2 * P]

@@ -510,7 +510,8 @@ def test_router_kernel(dtype, T, width, E, top):
 @pytest.mark.parametrize("T,width,ff,E,top,shared", [(1, 64, 32, 7, 3, True), (50, 48, 24, 5, 2, False),
                                                       (333, 128, 96, 6, 3, True), (17, 40, 20, 4, 4, True),
                                                       (5, 256, 64, 64, 1, False), (700, 96, 160, 3, 2, True),
-                                                      (900, 64, 96, 2, 2, False)])
+                                                      (900, 64, 96, 2, 2, False), (800, 128, 192, 4, 2, True),
+                                                      (300, 64, 64, 2, 2, False), (1000, 192, 320, 5, 3, True)])
 def test_experts_kernels(dtype, T, width, ff, E, top, shared):
     import torch_ops
     from qwen3_from_scratch_amd import ops
