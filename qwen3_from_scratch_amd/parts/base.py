@@ -160,6 +160,20 @@ class StreamAddend:
     bias: torch.Tensor = None
 
 
+@dataclass
+class HyperAddend:
+    """What a residual held in several streams still lacks: `values` (T, width) in the activation
+    dtype, a sublayer's result y, which enters every stream at once from the old ones,
+    x_t <- sum_s mix[s, t] x_s + write[t] * y, with `mix` (streams, streams) indexed [from, to] and
+    `write` (streams,), both float32 (a multiplier of the residual is part of `write`). A norm that
+    takes it as `delta` does this in float32 in the kernel that also reads the streams for the
+    next sublayer."""
+
+    values: torch.Tensor
+    mix: torch.Tensor
+    write: torch.Tensor
+
+
 def build_part(spec, prefix, precision, device):
     cls = lookup_part(spec.kind, spec.name)
     return cls(prefix=prefix, precision=precision, device=device, **dict(spec.params))

@@ -1,7 +1,9 @@
 """How a layer's parts are arranged around the residual stream."""
 
 from ..config.registry import register_part
-from .base import Part, UnscaledRows
+import torch
+
+from .base import HyperAddend, Part, TensorShape, UnscaledRows
 
 
 def _says(part, what):
@@ -96,3 +98,66 @@ class SandwichBlock(Part):
             return x, pending
         fed = self.feed_forward.forward(self.feed_forward_norm.forward(x, delta=pending), batch)
         return x, self._behind(self.feed_forward_out_norm, fed)
+
+
+@register_part("block", "hyper_connections")
+class HyperConnectionBlock(Part):
+    """A pre-norm layer over a residual that is held in `streams` copies x_1 .. x_n, (T, streams,
+    width) float32. Sublayer q (1: the mixer, 2: the feed-forward, which a layer may lack) has
+    three small tensors `hc<q>.in` (n), `hc<q>.out` (n) and `hc<q>.mix` (n, n), indexed [from, to]:
+
+        u = sum_s in[s] x_s,   y = sublayer(norm_q(u)),   x_t <- sum_s mix[s, t] x_s + mult out[t] y
+
+    for all t at once from the old streams. With `streams` 0 the layer has no such tensors and the
+    residual is the ordinary one, x <- x + mult y, which is the same computation with one stream,
+    in = out = mix = 1. The update of one sublayer and the read of the next are one kernel: what a
+    sublayer returns travels as a `HyperAddend` to the norm that reads the streams next (this
+    block's second, the next block's first, or the model's last, which reads their plain sum)."""
+
+    graph_safe = True
+
+    def __init__(self, prefix, precision, device, streams, mult=1.0):
+        super().__init__(prefix, precision, device)
+        self.streams, self.mult = int(streams), float(mult)
+        self.mixer = self.feed_forward = self.mixer_norm = self.feed_forward_norm = None
+        self.tables = {}
+
+    def attach(self, mixer, mixer_norm, feed_forward=None, feed_forward_norm=None):
+        if (feed_forward is None) != (feed_forward_norm is None):
+            raise ValueError("a feed-forward comes with its norm, or not at all")
+        self.mixer, self.mixer_norm = mixer, mixer_norm
+        self.feed_forward, self.feed_forward_norm = feed_forward, feed_forward_norm
+
+    def _sublayers(self):
+        return (1, 2) if self.feed_forward is not None else (1,)
+
+    def tensors(self):
+        names, n = {}, self.streams
+        if n:
+            for q in self._sublayers():
+                names[self._name("hc%d.in" % q)] = TensorShape((n,), "scale")
+                names[self._name("hc%d.out" % q)] = TensorShape((n,), "scale")
+                names[self._name("hc%d.mix" % q)] = TensorShape((n, n), "matrix")
+        return names
+
+    def load(self, fetch):
+        for q in self._sublayers():
+            if self.streams:
+                read = fetch(self._name("hc%d.in" % q), torch.float32).contiguous()
+                write = (fetch(self._name("hc%d.out" % q), torch.float32) * self.mult).contiguous()
+                mix = fetch(self._name("hc%d.mix" % q), torch.float32).contiguous()
+            else:
+                read = torch.ones(1, dtype=torch.float32, device=self.device)
+                write = torch.full((1,), self.mult, dtype=torch.float32, device=self.device)
+                mix = torch.ones((1, 1), dtype=torch.float32, device=self.device)
+            self.tables[q] = (read, write, mix)
+
+    def forward(self, x, pending, batch, cache, next_norm=None):
+        read, write, mix = self.tables[1]
+        y = self.mixer.forward(self.mixer_norm.forward(x, delta=pending, read=read), batch, cache)
+        pending = HyperAddend(y, mix, write)
+        if self.feed_forward is not None:
+            read, write, mix = self.tables[2]
+            y = self.feed_forward.forward(self.feed_forward_norm.forward(x, delta=pending, read=read), batch)
+            pending = HyperAddend(y, mix, write)
+        return x, pending

@@ -10,12 +10,14 @@ from .base import Part, StreamAddend, UnscaledRows
 @register_part("embedding", "token")
 class TokenEmbedding(Part):
     """x[t] = E[ids[t]], no scaling, no padding row
-    (src/qwen3_from_scratch/models/qwen3.py:17-19,45)."""
+    (src/qwen3_from_scratch/models/qwen3.py:17-19,45). With `copies` the residual starts as
+    that many equal streams, (T, copies, hidden_size), for blocks that keep several."""
 
     graph_safe = True
 
-    def __init__(self, prefix, precision, device, vocab_size, hidden_size, leaf="weight"):
+    def __init__(self, prefix, precision, device, vocab_size, hidden_size, leaf="weight", copies=0):
         super().__init__(prefix, precision, device)
+        self.copies = int(copies)
         self.vocab_size = vocab_size
         self.hidden_size = hidden_size
         self.leaf = leaf
@@ -28,6 +30,8 @@ class TokenEmbedding(Part):
         self.weight = fetch(self._name(self.leaf), self.precision.act)
 
     def forward(self, token_ids):
+        if self.copies:
+            return ops.embed_streams(token_ids, self.weight, self.copies)
         return ops.embed_rows(token_ids, self.weight)
 
 

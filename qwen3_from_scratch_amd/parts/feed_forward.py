@@ -20,8 +20,10 @@ class SwiGLU(Part):
     graph_safe = True
     feeds_sink = True
 
-    def __init__(self, prefix, precision, device, hidden_size, intermediate_size):
+    def __init__(self, prefix, precision, device, hidden_size, intermediate_size,
+                 names=("gate_proj.weight", "up_proj.weight", "down_proj.weight")):
         super().__init__(prefix, precision, device)
+        self.names = tuple(names)         # the tensors' names below the prefix: gate, up, down
         self.hidden_size = hidden_size
         self.intermediate_size = intermediate_size
         self.gate_up = None
@@ -29,20 +31,18 @@ class SwiGLU(Part):
 
     def tensors(self):
         H, I = self.hidden_size, self.intermediate_size
-        return {
-            self._name("gate_proj.weight"): (I, H),
-            self._name("up_proj.weight"): (I, H),
-            self._name("down_proj.weight"): (H, I),
-        }
+        gate, up, down = self.names
+        return {self._name(gate): (I, H), self._name(up): (I, H), self._name(down): (H, I)}
 
     def load(self, fetch):
         act = self.precision.act
         I, H = self.intermediate_size, self.hidden_size
         gate_up = torch.empty((2 * I, H), dtype=act, device=self.device)
-        gate_up[0::2].copy_(fetch(self._name("gate_proj.weight"), act, keep=False))
-        gate_up[1::2].copy_(fetch(self._name("up_proj.weight"), act, keep=False))
+        gate, up, down = self.names
+        gate_up[0::2].copy_(fetch(self._name(gate), act, keep=False))
+        gate_up[1::2].copy_(fetch(self._name(up), act, keep=False))
         self.gate_up = LinearWeight(gate_up, self.precision)
-        self.down = LinearWeight(fetch(self._name("down_proj.weight"), act), self.precision)
+        self.down = LinearWeight(fetch(self._name(down), act), self.precision)
 
     @property
     def takes_unscaled(self):

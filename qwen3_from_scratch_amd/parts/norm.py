@@ -4,7 +4,7 @@ import torch
 
 from .. import ops
 from ..config.registry import register_part
-from .base import NormSink, Part, StreamAddend, TensorShape
+from .base import HyperAddend, NormSink, Part, StreamAddend, TensorShape
 
 
 @register_part("norm", "rms")
@@ -56,3 +56,41 @@ class RMSNorm(Part):
         if not 1 <= rows <= ops.FUSED_ROWS_MOST or self.size % (16 if rows <= ops.FUSED_ROWS_FEW else 64):
             return None
         return NormSink(x, self.weight, self.eps, self.size)
+
+
+@register_part("norm", "layer")
+class LayerNorm(Part):
+    """y = (u - mean(u)) * rsqrt(var(u) + eps) * weight, var the mean of the squared deviations,
+    a weight and no bias. u is read from a float32 residual that is held in one or several
+    streams, (T, width) or (T, streams, width): u = sum_s read[s] x_s (`read` None: the plain sum,
+    which is also what the model's last norm wants). A `HyperAddend` given as `delta` first enters
+    all streams at once (x_t <- sum_s mix[s, t] x_s + write[t] y), a plain tensor is added to the
+    only stream; all of it float32 in one kernel, the result rounded once."""
+
+    graph_safe = True
+
+    def __init__(self, prefix, precision, device, size, eps, leaf="weight"):
+        super().__init__(prefix, precision, device)
+        self.size, self.eps, self.leaf = size, float(eps), leaf
+        self.weight = None
+        self._one = None
+
+    def tensors(self):
+        return {self._name(self.leaf): TensorShape((self.size,), "scale")}
+
+    def load(self, fetch):
+        self.weight = fetch(self._name(self.leaf))
+
+    def forward(self, x, delta=None, rows=None, read=None):
+        streams = x if x.dim() == 3 else x.unsqueeze(1)
+        mix = write = values = None
+        if isinstance(delta, HyperAddend):
+            values, mix, write = delta.values, delta.mix, delta.write
+        elif delta is not None:
+            if streams.shape[1] != 1:
+                raise ValueError("a plain addend joins a residual of one stream, not %d" % streams.shape[1])
+            if self._one is None:
+                self._one = torch.ones((1, 1), dtype=torch.float32, device=x.device)
+            values, mix, write = delta, self._one, self._one[0]
+        return ops.hyper_norm(streams, self.weight, self.eps, self.precision.act, read=read, delta=values, mix=mix,
+                              write=write, rows=rows, write_back=rows is None)

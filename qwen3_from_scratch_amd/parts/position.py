@@ -13,6 +13,18 @@ from ..config.registry import register_part
 from .base import Part
 
 
+def rotation_frequencies(dims, base, device):
+    """f_i = base^(-2i / dims), i < dims / 2, formed in double precision on the host and rounded
+    once to float32: what a mixer that carries its rotation among its own parameters hands to its
+    kernels, which form the angle as a float32 product of position and frequency. dims 0: None."""
+    if not dims:
+        return None
+    if dims % 2 or dims < 0:
+        raise ValueError("a rotation turns an even number of numbers, not %d" % dims)
+    freqs = [float(base) ** (-2.0 * i / dims) for i in range(dims // 2)]
+    return torch.tensor(freqs, dtype=torch.float64).to(torch.float32).to(device)
+
+
 @register_part("position", "none")
 class NoPosition(Part):
     graph_safe = True

@@ -296,7 +296,198 @@ def moe_experts(h, chosen, weights, up, down, shared=None, activation="erf"):
     return out.to(h.dtype)
 
 
+# ---- the recurrent mixers, the residual in several streams, attention with capped scores ----
+
+def embed_streams(ids, table, copies):
+    return table[ids.long()].float()[:, None, :].repeat(1, copies, 1).contiguous()
+
+
+def hyper_norm(x, weight, eps, out_dtype, read=None, delta=None, mix=None, write=None, rows=None, write_back=True):
+    src = x if rows is None else x[rows.long()]
+    if delta is not None:
+        d = (delta if rows is None else delta[rows.long()]).float()
+        src = torch.einsum("st,nsw->ntw", mix.float(), src) + write.float()[None, :, None] * d[:, None, :]
+        if write_back and rows is None:
+            x.copy_(src)
+    u = src.sum(dim=1) if read is None else torch.einsum("s,nsw->nw", read.float(), src)
+    if weight is None:
+        return None
+    dev = u - u.mean(dim=-1, keepdim=True)
+    var = (dev * dev).mean(dim=-1, keepdim=True)
+    return (dev * torch.rsqrt(var + eps) * weight.float()).to(out_dtype)
+
+
+def _sequences(cu_seqlens_q, slots):
+    cu = cu_seqlens_q.tolist()
+    return [(cu[b], cu[b + 1], int(slot)) for b, slot in enumerate(slots.tolist())]
+
+
+def causal_conv(x, weight, bias, state, slots, cu_seqlens_q, seq_index, activation=None, out_dtype=None, in_bias=None):
+    T, C = x.shape
+    taps = weight.shape[1]
+    out = torch.empty((T, C), dtype=torch.float32, device=x.device)
+    for first, last, slot in _sequences(cu_seqlens_q, slots):
+        if last == first:
+            continue
+        rows = x[first:last].float()
+        if in_bias is not None:
+            rows = rows + in_bias.float()
+        seen = torch.cat((state[slot].view(taps - 1, C), rows), dim=0)
+        acc = bias.float().expand(last - first, C).clone()
+        for j in range(taps):
+            acc += weight[:, taps - 1 - j].float() * seen[taps - 1 - j: taps - 1 - j + last - first]
+        out[first:last] = acc
+        state[slot] = seen[seen.shape[0] - (taps - 1):].reshape(-1)
+    if activation == "silu":
+        out = out * torch.sigmoid(out)
+    return out.to(out_dtype or x.dtype)
+
+
+def mamba2_scan(xbc, dt, dt_bias, a_log, d_skip, state, slots, cu_seqlens_q, heads, vdim, n_state, groups):
+    T = xbc.shape[0]
+    inner, gn = heads * vdim, groups * n_state
+    x = xbc[:, :inner].float().view(T, heads, vdim)
+    B = xbc[:, inner:inner + gn].float().view(T, groups, n_state).repeat_interleave(heads // groups, dim=1)
+    C = xbc[:, inner + gn:].float().view(T, groups, n_state).repeat_interleave(heads // groups, dim=1)
+    step = torch.nn.functional.softplus(dt.float() + dt_bias.float())
+    decay = torch.exp(-torch.exp(a_log.float()) * step)
+    y = torch.empty((T, heads, vdim), dtype=torch.float32, device=xbc.device)
+    for first, last, slot in _sequences(cu_seqlens_q, slots):
+        S = state[slot].view(heads, n_state, vdim).clone()
+        for t in range(first, last):
+            S = decay[t][:, None, None] * S + step[t][:, None, None] * B[t][:, :, None] * x[t][:, None, :]
+            y[t] = torch.einsum("hnp,hn->hp", S, C[t]) + d_skip.float()[:, None] * x[t]
+        state[slot] = S.reshape(-1)
+    return y.view(T, inner)
+
+
+def gated_rmsnorm(y, gate, weight, groups, eps, out_dtype):
+    T, inner = y.shape
+    g = gate.float()
+    v = (y.float() * g * torch.sigmoid(g)).view(T, groups, inner // groups)
+    v = v * torch.rsqrt((v * v).mean(dim=-1, keepdim=True) + eps)
+    return (v.view(T, inner) * weight.float()).to(out_dtype)
+
+
+def block_gates(u, weights, biases):
+    T, width = u.shape
+    blocks = weights.shape[1]
+    ub = u.float().view(T, blocks, width // blocks)
+    z = torch.einsum("tbi,gbio->gtbo", ub, weights.float()) + biases.float()[:, None]
+    return torch.sigmoid(z).reshape(2, T, width)
+
+
+def rglru_scan(u, gates, rate, y, y_bias, state, slots, cu_seqlens_q, out_dtype):
+    T, width = u.shape
+    a = torch.exp(-rate.float() * gates[0])
+    push = torch.sqrt(1.0 - a * a) * gates[1] * u.float()
+    z = y.float() + y_bias.float()
+    branch = 0.5 * z * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * z ** 3)))
+    out = torch.empty((T, width), dtype=torch.float32, device=u.device)
+    for first, last, slot in _sequences(cu_seqlens_q, slots):
+        S = state[slot].clone()
+        for t in range(first, last):
+            S = a[t] * S + push[t]
+            out[t] = S * branch[t]
+        state[slot] = S
+    return out.to(out_dtype)
+
+
+def _turn(v, positions, inv_freq, neighbours):
+    """v (T, heads, dim): the first 2 * len(inv_freq) numbers of each head turn by position * frequency,
+    pairs (2i, 2i + 1) or (i, i + half)."""
+    if inv_freq is None:
+        return v
+    half = inv_freq.shape[0]
+    ang = positions.float()[:, None] * inv_freq.float()[None, :]
+    c, s = ang.cos()[:, None, :], ang.sin()[:, None, :]
+    out = v.clone()
+    if neighbours:
+        a, b = v[..., 0:2 * half:2], v[..., 1:2 * half:2]
+        out[..., 0:2 * half:2] = a * c - b * s
+        out[..., 1:2 * half:2] = b * c + a * s
+    else:
+        a, b = v[..., :half], v[..., half:2 * half]
+        out[..., :half] = a * c - b * s
+        out[..., half:2 * half] = b * c + a * s
+    return out
+
+
+def retention_scan(qkvg, heads, dim, vdim, inv_freq, positions, decay, k_scale, eps, state, slots, cu_seqlens_q, out_dtype):
+    T = qkvg.shape[0]
+    hd, hv = heads * dim, heads * vdim
+    rows = qkvg.float()
+    q = _turn(rows[:, :hd].view(T, heads, dim), positions, inv_freq, False)
+    k = _turn(rows[:, hd:2 * hd].view(T, heads, dim), positions, inv_freq, False) * k_scale
+    v = rows[:, 2 * hd:2 * hd + hv].view(T, heads, vdim)
+    g = rows[:, 2 * hd + hv:]
+    o = torch.empty((T, heads, vdim), dtype=torch.float32, device=qkvg.device)
+    for first, last, slot in _sequences(cu_seqlens_q, slots):
+        S = state[slot].view(heads, dim, vdim).clone()
+        for t in range(first, last):
+            S = decay.float()[:, None, None] * S + k[t][:, :, None] * v[t][:, None, :]
+            o[t] = torch.einsum("hdv,hd->hv", S, q[t])
+        state[slot] = S.reshape(-1)
+    o = o * torch.rsqrt((o * o).mean(dim=-1, keepdim=True) + eps)
+    return (o.reshape(T, hv) * g * torch.sigmoid(g)).to(out_dtype)
+
+
+def softcap_prepare(rows, bias, heads, kv_heads, dim, vdim, q_weight, k_weight, eps, inv_freq, positions, seq_index,
+                    out_dtype, block_table=None, k_cache=None, v_cache=None):
+    T = rows.shape[0]
+    nq, nk, nv = heads * dim, kv_heads * dim, kv_heads * vdim
+    z = rows[:, :nq + nk + nv].float() + bias.float()
+    q, k, v = z[:, :nq], z[:, nq:nq + nk], z[:, nq + nk:]
+    q = q * torch.rsqrt((q * q).mean(dim=-1, keepdim=True) + eps) * q_weight.float()
+    k = k * torch.rsqrt((k * k).mean(dim=-1, keepdim=True) + eps) * k_weight.float()
+    q = _turn(q.view(T, heads, dim), positions, inv_freq, True)
+    k = _turn(k.view(T, kv_heads, dim), positions, inv_freq, True)
+    if k_cache is not None:
+        page = k_cache.shape[2]
+        pos = positions.long()
+        pages = block_table[seq_index.long(), pos // page].long()
+        k_cache[pages, :, pos % page] = k.to(k_cache.dtype)
+        v_cache[pages, :, pos % page] = v.reshape(T, kv_heads, vdim).to(v_cache.dtype)
+    return q.to(out_dtype).contiguous()
+
+
+def softcap_attention(q, k_cache, v_cache, block_table, cu_seqlens_q, kv_lens, seq_index, positions, max_q_len,
+                      max_kv_len, scale, softcap, window=0, gate=None):
+    T, H, dim = q.shape
+    G, page, vdim = k_cache.shape[1], k_cache.shape[2], v_cache.shape[3]
+    res = torch.zeros((T, H, vdim), dtype=torch.float32, device=q.device)
+    cu, kvl = cu_seqlens_q.tolist(), kv_lens.tolist()
+    for b in range(len(kvl)):
+        q0, q1, L = cu[b], cu[b + 1], kvl[b]
+        n = q1 - q0
+        if n == 0:
+            continue
+        blocks = -(-L // page)
+        pages = block_table[b, :blocks].long().clamp(min=0)
+        K = k_cache[pages].float().permute(1, 0, 2, 3).reshape(G, blocks * page, dim)[:, :L]
+        V = v_cache[pages].float().permute(1, 0, 2, 3).reshape(G, blocks * page, vdim)[:, :L]
+        qpos = torch.arange(L - n, L, device=q.device)[:, None]
+        kpos = torch.arange(L, device=q.device)[None, :]
+        hidden = kpos > qpos
+        if window > 0:
+            hidden = hidden | (qpos - kpos >= window)
+        for h in range(H):
+            s = (q[q0:q1, h].float() @ K[h // (H // G)].T) * scale
+            if softcap > 0:
+                s = softcap * torch.tanh(s / softcap)
+            s = s.masked_fill(hidden, float("-inf"))
+            res[q0:q1, h] = torch.softmax(s, dim=-1) @ V[h // (H // G)]
+    if gate is not None:
+        res = res * torch.sigmoid(gate.float())[:, :, None]
+    return res.reshape(T, H * vdim).to(q.dtype)
+
+
+def scaled_sum(a, alpha, b, beta):
+    return (alpha * a.float() + beta * b.float()).to(a.dtype)
+
+
 ALL = ("embed_rows", "swiglu", "rmsnorm", "rope_table", "qk_norm_rope_store",
        "paged_attention", "decode_attention_takes", "linear", "linear_swiglu", "tile_weight", "sample",
        "rmsnorm_addend", "gelu", "GELU_KINDS", "latent_prepare", "headwise_linear", "rotate_heads", "latent_attention",
-       "moe_route", "moe_experts")
+       "moe_route", "moe_experts", "embed_streams", "hyper_norm", "causal_conv", "mamba2_scan", "gated_rmsnorm",
+       "block_gates", "rglru_scan", "retention_scan", "softcap_prepare", "softcap_attention", "scaled_sum")
