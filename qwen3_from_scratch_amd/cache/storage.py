@@ -59,6 +59,19 @@ class CacheStorage:
             for t in self.states:
                 t[:, index] = 0
 
+    def keep_states(self, slots):
+        """Copies of the states in `slots` (a device tensor of slot numbers), to be put back by
+        `put_states`: a step that is run for another reason than its result (the eager run before a
+        graph is captured) must leave no trace in states that the real step then continues. Pages
+        need no such care: the real step writes the same keys to the same places again."""
+        index = slots.long()
+        return index, [t.index_select(1, index) for t in self.states]
+
+    def put_states(self, kept):
+        index, copies = kept
+        for t, copy in zip(self.states, copies):
+            t.index_copy_(1, index, copy)
+
     def bind(self, block_tables):
         """`block_tables`: per paged group the step's int32 (B, W) device tensor."""
         self._block_tables = block_tables

@@ -158,7 +158,10 @@ class _DecodeGraph:
         side = torch.cuda.Stream(device=runner.device)
         side.wait_stream(torch.cuda.current_stream(runner.device))
         with torch.cuda.stream(side):
+            # mixers with a recurrent state would otherwise take this step's tokens twice
+            kept = runner.storage.keep_states(batch.state_slots)
             runner.model.forward(batch, runner.storage)
+            runner.storage.put_states(kept)
         torch.cuda.current_stream(runner.device).wait_stream(side)
         torch.cuda.synchronize(runner.device)
         graph = torch.cuda.CUDAGraph()

@@ -38,6 +38,17 @@ __all__ = [
     "latent_attention",
     "moe_route",
     "moe_experts",
+    "embed_streams",
+    "hyper_norm",
+    "causal_conv",
+    "mamba2_scan",
+    "gated_rmsnorm",
+    "block_gates",
+    "rglru_scan",
+    "retention_scan",
+    "softcap_prepare",
+    "softcap_attention",
+    "scaled_sum",
     "linear",
     "linear_plain",
     "linear_swiglu",
@@ -556,6 +567,308 @@ def moe_experts(h, chosen, weights, up, down, shared=None, activation="erf"):
                                  _DT[h.dtype], stream), "moe_linear")
     _check(lib.q3_moe_combine(_ptr(y), _ptr(slot_of_pair), _ptr(weights), _ptr(shared), _ptr(out), T, width, top,
                               _DT[h.dtype], stream), "moe_combine")
+    return out
+
+
+# ---- a residual in several streams; the recurrent mixers; attention with capped scores ----
+
+def _f32(t, shape, what):
+    _need(t.dtype == torch.float32 and tuple(t.shape) == tuple(shape) and t.is_contiguous() and t.is_cuda,
+          "%s must be float32 %s on the GPU, contiguous" % (what, tuple(shape)))
+
+
+def _rows_view(t, what):
+    """A 2-D tensor whose rows may lie apart (a stretch of columns of a wider tensor)."""
+    _need(t.is_cuda and t.dim() == 2 and (t.shape[1] == 1 or t.stride(1) == 1) and t.dtype in _DT,
+          "%s must be (rows, n) on the GPU with its columns side by side" % what)
+    return t.stride(0)
+
+
+def _sequences(slots, cu_seqlens_q, state, numbers, what):
+    _need(slots.dtype == torch.int32 and cu_seqlens_q.dtype == torch.int32 and slots.dim() == 1
+          and cu_seqlens_q.shape == (slots.shape[0] + 1,), "slots int32 (B,), cu_seqlens_q int32 (B + 1,)")
+    _dev(slots, cu_seqlens_q)
+    _need(state.is_cuda and state.dtype == torch.float32 and state.dim() == 2 and state.shape[1] == numbers
+          and (numbers == 1 or state.stride(1) == 1),
+          "%s: the state must be float32 (slots, %d) on the GPU with its columns side by side" % (what, numbers))
+    return slots.shape[0]
+
+
+def embed_streams(ids, table, copies):
+    """out[t, s, :] = float32(table[ids[t], :]) for s < copies: a residual that starts as equal streams."""
+    _dev(ids, table)
+    _need(ids.dtype == torch.int32 and ids.dim() == 1, "ids must be int32 (T,)")
+    _need(table.dim() == 2 and table.dtype in _DT and 1 <= copies <= 8, "table (V, W) bfloat16 or float32; 1 to 8 copies")
+    T, (V, W) = ids.shape[0], table.shape
+    out = torch.empty((T, copies, W), dtype=torch.float32, device=table.device)
+    if T:
+        _check(library("hyper").q3_embed_streams(_ptr(ids), _ptr(table), _ptr(out), T, copies, W, V, _DT[table.dtype],
+                                                 _stream()), "embed_streams")
+    return out
+
+
+def hyper_norm(x, weight, eps, out_dtype, read=None, delta=None, mix=None, write=None, rows=None, write_back=True):
+    """Layer norm of a float32 residual held in streams, x (T, S, W), behind an addend that enters
+    all streams at once. For each output row r (source row s = rows[r], or r):
+
+    with `delta` (T, W, activation dtype), `mix` (S, S) indexed [from, to] and `write` (S,):
+    x[s, t] <- sum_f mix[f, t] x[s, f] + write[t] * delta[s] for all t from the old streams, stored if
+    `write_back` and `rows` is None; u = sum_f read[f] x[s, f] (`read` None: the plain sum);
+    out[r] = (u - mean(u)) * rsqrt(mean((u - mean(u))^2) + eps) * weight, rounded once to `out_dtype`.
+    With `weight` None only the streams are brought up to date and None is returned."""
+    _dev(x, weight, delta, mix, write, read, rows)
+    _need(x.dim() == 3 and x.dtype == torch.float32 and 1 <= x.shape[1] <= 8, "x must be float32 (T, S, W), S at most 8")
+    T, S, W = x.shape
+    _need(out_dtype in _DT, "out_dtype must be bfloat16 or float32")
+    if weight is not None:
+        _f32(weight, (W,), "weight")
+    if read is not None:
+        _f32(read, (S,), "read")
+    if delta is not None:
+        _need(delta.shape == (T, W) and delta.dtype == out_dtype, "delta must be (T, W) of the activation dtype")
+        _need(mix is not None and write is not None, "a delta comes with mix and write")
+        _f32(mix, (S, S), "mix")
+        _f32(write, (S,), "write")
+    n_out = T
+    if rows is not None:
+        _need(rows.dtype == torch.int32 and rows.dim() == 1, "rows must be int32 (R,)")
+        n_out = rows.shape[0]
+    _need(weight is not None or rows is None, "without a weight there is no output")
+    out = torch.empty((n_out, W), dtype=out_dtype, device=x.device) if weight is not None else None
+    if n_out:
+        _check(library("hyper").q3_hyper_norm(
+            _ptr(x), _ptr(delta), _ptr(mix), _ptr(write), _ptr(read), _ptr(weight), _ptr(rows), _ptr(out), n_out, S, W,
+            ctypes.c_float(eps), _DT[out_dtype], 1 if (write_back and rows is None and delta is not None) else 0,
+            _stream()), "hyper_norm")
+    return out
+
+
+def causal_conv(x, weight, bias, state, slots, cu_seqlens_q, seq_index, activation=None, out_dtype=None, in_bias=None):
+    """A causal convolution per channel over a packed step, continued from each sequence's state.
+
+    x (T, C), rows possibly apart; weight float32 (C, taps), the last tap the current token's; bias
+    float32 (C,); `in_bias` float32 (C,) is added to x first. state float32 (slots, (taps - 1) * C):
+    a sequence's last taps - 1 inputs, oldest first (zeros for a fresh sequence), brought up to
+    date. `activation`: None or "silu". Returns (T, C) of `out_dtype` (x's by default)."""
+    stride = _rows_view(x, "x")
+    T, C = x.shape
+    taps = weight.shape[1] if weight.dim() == 2 else 0
+    _f32(weight, (C, taps), "weight")
+    _f32(bias, (C,), "bias")
+    if in_bias is not None:
+        _f32(in_bias, (C,), "in_bias")
+    _need(1 <= taps <= 8 and activation in (None, "silu"), "1 to 8 taps; activation None or silu")
+    B = _sequences(slots, cu_seqlens_q, state, (taps - 1) * C, "causal_conv")
+    _need(seq_index.dtype == torch.int32 and seq_index.shape == (T,), "seq_index must be int32 (T,)")
+    _dev(seq_index)
+    out_dtype = out_dtype or x.dtype
+    _need(out_dtype in _DT, "out_dtype must be bfloat16 or float32")
+    out = torch.empty((T, C), dtype=out_dtype, device=x.device)
+    if T:
+        _check(library("recurrent").q3_causal_conv(
+            _ptr(x), ctypes.c_long(stride), _ptr(in_bias), _ptr(weight), _ptr(bias), _ptr(state),
+            ctypes.c_long(state.stride(0)), _ptr(slots), _ptr(cu_seqlens_q), _ptr(seq_index), _ptr(out), T, B, C, taps,
+            1 if activation == "silu" else 0, _DT[x.dtype], _DT[out_dtype], _stream()), "causal_conv")
+    return out
+
+
+def mamba2_scan(xbc, dt, dt_bias, a_log, d_skip, state, slots, cu_seqlens_q, heads, vdim, n_state, groups):
+    """The Mamba-2 recurrence over a packed step. xbc (T, heads vdim + 2 groups n_state), contiguous,
+    rows [x | B | C]; dt (T, heads), rows possibly apart, same dtype; dt_bias, a_log, d_skip float32
+    (heads,). Per head h of group g = h // (heads / groups), with step = softplus(dt + dt_bias):
+    S <- exp(-exp(a_log) step) S + step B x^T, y = S^T C + d_skip x. state float32 (slots,
+    heads n_state vdim) laid out (head, n, column), continued and brought up to date. Returns y
+    float32 (T, heads vdim)."""
+    _dev(xbc, dt_bias, a_log, d_skip)
+    T = xbc.shape[0]
+    _need(xbc.dim() == 2 and xbc.dtype in _DT and xbc.shape[1] == heads * vdim + 2 * groups * n_state,
+          "xbc must be (T, heads vdim + 2 groups n_state)")
+    stride = _rows_view(dt, "dt")
+    _need(dt.shape == (T, heads) and dt.dtype == xbc.dtype, "dt must be (T, heads) of xbc's dtype")
+    for t, what in ((dt_bias, "dt_bias"), (a_log, "a_log"), (d_skip, "d_skip")):
+        _f32(t, (heads,), what)
+    _need(heads % groups == 0 and n_state <= 256, "groups must divide heads; n_state at most 256")
+    B = _sequences(slots, cu_seqlens_q, state, heads * n_state * vdim, "mamba2_scan")
+    y = torch.empty((T, heads * vdim), dtype=torch.float32, device=xbc.device)
+    if T:
+        _check(library("recurrent").q3_mamba2_scan(
+            _ptr(xbc), _ptr(dt), ctypes.c_long(stride), _ptr(dt_bias), _ptr(a_log), _ptr(d_skip), _ptr(state),
+            ctypes.c_long(state.stride(0)), _ptr(slots), _ptr(cu_seqlens_q), _ptr(y), B, heads, vdim, n_state, groups,
+            _DT[xbc.dtype], _stream()), "mamba2_scan")
+    return y
+
+
+def gated_rmsnorm(y, gate, weight, groups, eps, out_dtype):
+    """v = y * silu(gate); out = v * rsqrt(mean(v^2) + eps) * weight, the mean taken over each of
+    `groups` equal parts of a row. y float32 (T, n) contiguous, gate (T, n) of `out_dtype`, rows
+    possibly apart, weight float32 (n,)."""
+    _dev(y, weight)
+    _need(y.dim() == 2 and y.dtype == torch.float32, "y must be float32 (T, n)")
+    T, n = y.shape
+    stride = _rows_view(gate, "gate")
+    _need(gate.shape == (T, n) and gate.dtype == out_dtype and out_dtype in _DT, "gate must be (T, n) of out_dtype")
+    _f32(weight, (n,), "weight")
+    _need(groups >= 1 and n % groups == 0, "groups must divide the row")
+    out = torch.empty((T, n), dtype=out_dtype, device=y.device)
+    if T:
+        _check(library("hyper").q3_gated_rmsnorm(_ptr(y), _ptr(gate), ctypes.c_long(stride), _ptr(weight), _ptr(out), T, n,
+                                                 groups, ctypes.c_float(eps), _DT[out_dtype], _stream()), "gated_rmsnorm")
+    return out
+
+
+def block_gates(u, weights, biases):
+    """out[g, t, b bw + o] = sigmoid(biases[g, b, o] + sum_i weights[g, b, i, o] u[t, b bw + i]): two gates
+    from block-diagonal matrices, float32 throughout. u (T, width), weights (2, blocks, bw, bw) indexed
+    (gate, block, in, out), biases (2, blocks, bw). Returns (2, T, width)."""
+    _dev(u, weights, biases)
+    _need(u.dim() == 2 and u.dtype == torch.float32, "u must be float32 (T, width)")
+    T, width = u.shape
+    _need(weights.dim() == 4 and weights.shape[0] == 2 and weights.shape[2] == weights.shape[3]
+          and weights.shape[1] * weights.shape[2] == width, "weights must be (2, blocks, bw, bw) with blocks bw = width")
+    blocks, bw = weights.shape[1], weights.shape[2]
+    _f32(weights, (2, blocks, bw, bw), "weights")
+    _f32(biases, (2, blocks, bw), "biases")
+    out = torch.empty((2, T, width), dtype=torch.float32, device=u.device)
+    if T:
+        _check(library("recurrent").q3_block_gates(_ptr(u), _ptr(weights), _ptr(biases), _ptr(out), T, width, blocks,
+                                                   _stream()), "block_gates")
+    return out
+
+
+def rglru_scan(u, gates, rate, y, y_bias, state, slots, cu_seqlens_q, out_dtype):
+    """The real-gated linear recurrence over a packed step, float32: with r = gates[0], i = gates[1],
+    a = exp(-rate r): S <- a S + sqrt(1 - a^2) i u; out = S * gelu_tanh(y + y_bias), rounded once to
+    `out_dtype`. u (T, width) and gates (2, T, width) float32 contiguous, y float32 (T, width) with
+    rows possibly apart, rate and y_bias float32 (width,), state float32 (slots, width)."""
+    _dev(u, gates, rate, y_bias)
+    _need(u.dim() == 2 and u.dtype == torch.float32, "u must be float32 (T, width)")
+    T, width = u.shape
+    _f32(gates, (2, T, width), "gates")
+    _f32(rate, (width,), "rate")
+    _f32(y_bias, (width,), "y_bias")
+    stride = _rows_view(y, "y")
+    _need(y.shape == (T, width) and y.dtype == torch.float32 and out_dtype in _DT, "y must be float32 (T, width)")
+    B = _sequences(slots, cu_seqlens_q, state, width, "rglru_scan")
+    out = torch.empty((T, width), dtype=out_dtype, device=u.device)
+    if T:
+        _check(library("recurrent").q3_rglru_scan(
+            _ptr(u), _ptr(gates), _ptr(rate), _ptr(y), ctypes.c_long(stride), _ptr(y_bias), _ptr(state),
+            ctypes.c_long(state.stride(0)), _ptr(slots), _ptr(cu_seqlens_q), _ptr(out), T, B, width, _DT[out_dtype],
+            _stream()), "rglru_scan")
+    return out
+
+
+def retention_scan(qkvg, heads, dim, vdim, inv_freq, positions, decay, k_scale, eps, state, slots, cu_seqlens_q, out_dtype):
+    """Retention over a packed step. qkvg (T, 2 heads dim + 2 heads vdim) contiguous, rows
+    [q | k | v | g]. q and k turn by the position over their first 2 len(inv_freq) numbers, pairs
+    (i, i + len(inv_freq)), angle = position * inv_freq[i] in float32 (`inv_freq` None: no rotation);
+    k is multiplied by `k_scale`. Per head S <- decay S + k v^T, o = S^T q; o is divided by the root
+    mean square of the head's vdim numbers (eps inside the root) and multiplied by silu(g). state
+    float32 (slots, heads dim vdim) laid out (head, dim, column). Returns (T, heads vdim)."""
+    _dev(qkvg, inv_freq, positions, decay)
+    T = qkvg.shape[0]
+    _need(qkvg.dim() == 2 and qkvg.dtype in _DT and qkvg.dtype == out_dtype
+          and qkvg.shape[1] == 2 * heads * dim + 2 * heads * vdim, "qkvg must be (T, 2 heads dim + 2 heads vdim) of out_dtype")
+    half = 0
+    if inv_freq is not None:
+        half = inv_freq.shape[0]
+        _f32(inv_freq, (half,), "inv_freq")
+    _need(2 * half <= dim and dim <= 256 and vdim <= 1024, "the rotation fits the head; dim at most 256, vdim at most 1024")
+    _need(positions.dtype == torch.int32 and positions.shape == (T,), "positions must be int32 (T,)")
+    _f32(decay, (heads,), "decay")
+    B = _sequences(slots, cu_seqlens_q, state, heads * dim * vdim, "retention_scan")
+    out = torch.empty((T, heads * vdim), dtype=out_dtype, device=qkvg.device)
+    if T:
+        _check(library("recurrent").q3_retention_scan(
+            _ptr(qkvg), _ptr(inv_freq), half, _ptr(positions), _ptr(decay), ctypes.c_float(k_scale), ctypes.c_float(eps),
+            _ptr(state), ctypes.c_long(state.stride(0)), _ptr(slots), _ptr(cu_seqlens_q), _ptr(out), B, heads, dim, vdim,
+            _DT[out_dtype], _stream()), "retention_scan")
+    return out
+
+
+def softcap_prepare(rows, bias, heads, kv_heads, dim, vdim, q_weight, k_weight, eps, inv_freq, positions, seq_index,
+                    out_dtype, block_table=None, k_cache=None, v_cache=None):
+    """Queries, keys and values of a step from the float32 rows of their joint product.
+
+    rows float32 (T, n), n >= heads dim + kv_heads dim + kv_heads vdim, laid out [q | k | v | ...];
+    bias float32 over q, k and v is added; q and k are each divided by the root mean square of the
+    whole projection and multiplied by `q_weight` (heads dim) and `k_weight` (kv_heads dim); the
+    first 2 len(inv_freq) numbers of every head turn in pairs (2i, 2i + 1) by position * inv_freq[i].
+    Returns q (T, heads, dim) of `out_dtype`; with a cache, keys (pages, kv_heads, page, dim) and
+    values (pages, kv_heads, page, vdim) receive the tokens at their positions."""
+    _dev(bias, q_weight, k_weight, inv_freq, positions, seq_index, block_table, k_cache, v_cache)
+    _need(rows.is_cuda and rows.dim() == 2 and rows.dtype == torch.float32 and rows.stride(1) == 1, "rows must be float32 (T, n)")
+    T = rows.shape[0]
+    nq, nk, nv = heads * dim, kv_heads * dim, kv_heads * vdim
+    _need(rows.shape[1] >= nq + nk + nv and heads % kv_heads == 0, "rows hold q, k and v; kv_heads divides heads")
+    _f32(bias, (nq + nk + nv,), "bias")
+    _f32(q_weight, (nq,), "q_weight")
+    _f32(k_weight, (nk,), "k_weight")
+    half = 0
+    if inv_freq is not None:
+        half = inv_freq.shape[0]
+        _f32(inv_freq, (half,), "inv_freq")
+    _need(2 * half <= dim and out_dtype in _DT, "the rotation fits the head")
+    _need(positions.dtype == torch.int32 and positions.shape == (T,) and seq_index.dtype == torch.int32
+          and seq_index.shape == (T,), "positions and seq_index must be int32 (T,)")
+    page = width = 0
+    if k_cache is not None:
+        _need(v_cache is not None and block_table is not None and block_table.dtype == torch.int32 and block_table.dim() == 2,
+              "a key cache comes with a value cache and an int32 block table")
+        page, width = k_cache.shape[2], block_table.shape[1]
+        _need(k_cache.dim() == 4 and k_cache.shape[1:] == (kv_heads, page, dim) and v_cache.dim() == 4
+              and v_cache.shape[1:] == (kv_heads, page, vdim) and k_cache.dtype == out_dtype and v_cache.dtype == out_dtype,
+              "keys (pages, kv_heads, page, dim) and values (pages, kv_heads, page, vdim) of out_dtype")
+    q = torch.empty((T, heads, dim), dtype=out_dtype, device=rows.device)
+    if T:
+        _check(library("softcap").q3_softcap_prepare(
+            _ptr(rows), ctypes.c_long(rows.stride(0)), _ptr(bias), _ptr(q_weight), _ptr(k_weight), ctypes.c_float(eps),
+            _ptr(inv_freq), half, _ptr(positions), _ptr(seq_index), _ptr(block_table), width, _ptr(k_cache), _ptr(v_cache),
+            page, _ptr(q), T, heads, kv_heads, dim, vdim, _DT[out_dtype], _stream()), "softcap_prepare")
+    return q
+
+
+def softcap_attention(q, k_cache, v_cache, block_table, cu_seqlens_q, kv_lens, seq_index, positions, max_q_len,
+                      max_kv_len, scale, softcap, window=0, gate=None):
+    """Causal softmax attention over a paged cache whose keys and values differ in size.
+
+    q (T, heads, dim); keys (pages, kv_heads, page, dim), values (pages, kv_heads, page, vdim); the
+    token at row t of sequence seq_index[t] sits at positions[t] and sees the keys at positions
+    j <= positions[t] (with `window` > 0 only the last `window` of them). score = (q . k) scale, then
+    softcap * tanh(score / softcap) if softcap > 0; softmax in float32. `gate` float32 (T, heads),
+    rows possibly apart: head h's result is multiplied by sigmoid(gate[t, h]). Returns (T, heads vdim)."""
+    _dev(q, k_cache, v_cache, block_table, seq_index, positions)
+    _need(q.dim() == 3 and q.dtype in _DT, "q must be (T, heads, dim)")
+    T, H, dim = q.shape
+    _need(k_cache.dim() == 4 and v_cache.dim() == 4 and k_cache.shape[3] == dim and k_cache.shape[:3] == v_cache.shape[:3]
+          and k_cache.dtype == q.dtype and v_cache.dtype == q.dtype, "keys (pages, G, page, dim), values (pages, G, page, vdim)")
+    G, page, vdim = k_cache.shape[1], k_cache.shape[2], v_cache.shape[3]
+    _need(H % G == 0 and dim <= 512 and vdim <= 512, "kv heads divide heads; dim and vdim at most 512")
+    _need(block_table.dtype == torch.int32 and block_table.dim() == 2, "block_table must be int32 (B, W)")
+    _need(positions.dtype == torch.int32 and positions.shape == (T,) and seq_index.dtype == torch.int32
+          and seq_index.shape == (T,), "positions and seq_index must be int32 (T,)")
+    _need(max_kv_len <= block_table.shape[1] * page, "the block table does not cover the longest sequence")
+    stride = 0
+    if gate is not None:
+        stride = _rows_view(gate, "gate")
+        _need(gate.shape == (T, H) and gate.dtype == torch.float32, "gate must be float32 (T, heads)")
+    out = torch.empty((T, H * vdim), dtype=q.dtype, device=q.device)
+    if T:
+        _check(library("softcap").q3_softcap_attention(
+            _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(seq_index),
+            _ptr(positions), ctypes.c_float(scale), ctypes.c_float(softcap), int(window), _ptr(gate),
+            ctypes.c_long(stride), _ptr(out), T, H, G, dim, vdim, page, _DT[q.dtype], _stream()), "softcap_attention")
+    return out
+
+
+def scaled_sum(a, alpha, b, beta):
+    """alpha * a + beta * b, elementwise in float32, rounded once to the operands' dtype."""
+    _dev(a, b)
+    _need(a.shape == b.shape and a.dtype == b.dtype and a.dtype in _DT, "a and b must be alike, bfloat16 or float32")
+    out = torch.empty_like(a)
+    if a.numel():
+        _check(library("hyper").q3_scaled_sum(_ptr(a), ctypes.c_float(alpha), _ptr(b), ctypes.c_float(beta), _ptr(out),
+                                              ctypes.c_long(a.numel()), _DT[a.dtype], _stream()), "scaled_sum")
     return out
 
 

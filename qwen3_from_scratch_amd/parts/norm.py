@@ -79,7 +79,7 @@ class LayerNorm(Part):
         return {self._name(self.leaf): TensorShape((self.size,), "scale")}
 
     def load(self, fetch):
-        self.weight = fetch(self._name(self.leaf))
+        self.weight = fetch(self._name(self.leaf), torch.float32)
 
     def forward(self, x, delta=None, rows=None, read=None):
         streams = x if x.dim() == 3 else x.unsqueeze(1)
