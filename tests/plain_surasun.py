@@ -134,8 +134,9 @@ def softcap_attention(h, w, p, m, eps):
     v = (h @ _t(w, p + "v").T + _t(w, p + "v.b")).reshape(T, G, dv)
     q = (rms_unit(q, eps) * _t(w, p + "q.norm")).reshape(T, H, d)
     k = (rms_unit(k, eps) * _t(w, p + "k.norm")).reshape(T, G, d)
-    q = turn_neighbours(q, pos, m["rot"]["dims"], m["rot"]["base"])
-    k = turn_neighbours(k, pos, m["rot"]["dims"], m["rot"]["base"])
+    if m.get("rot"):
+        q = turn_neighbours(q, pos, m["rot"]["dims"], m["rot"]["base"])
+        k = turn_neighbours(k, pos, m["rot"]["dims"], m["rot"]["base"])
     gate = torch.sigmoid(h @ _t(w, p + "g").T)
     cap = m.get("softcap")
     out = torch.zeros(T, H, dv, dtype=F)
@@ -153,8 +154,11 @@ def retention(h, w, p, m, eps):
     T = h.shape[0]
     H, d, dv = m["heads"], m["dim"], m["vdim"]
     pos = torch.arange(T)
-    q = turn_halves((h @ _t(w, p + "q").T).reshape(T, H, d), pos, m["rot"]["dims"], m["rot"]["base"])
-    k = turn_halves((h @ _t(w, p + "k").T).reshape(T, H, d), pos, m["rot"]["dims"], m["rot"]["base"]) * d ** -0.5
+    q, k = (h @ _t(w, p + "q").T).reshape(T, H, d), (h @ _t(w, p + "k").T).reshape(T, H, d)
+    if m.get("rot"):
+        q = turn_halves(q, pos, m["rot"]["dims"], m["rot"]["base"])
+        k = turn_halves(k, pos, m["rot"]["dims"], m["rot"]["base"])
+    k = k * d ** -0.5
     v = (h @ _t(w, p + "v").T).reshape(T, H, dv)
     o = torch.zeros(T, H, dv, dtype=F)
     S = torch.zeros(H, d, dv, dtype=F)
