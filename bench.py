@@ -2,7 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--layers L]
                     [--shape 8b|14b|32b|0.6b] [--prompt P] [--context C]
-                    [--workload decode|continuous|served|prefix|products|kodisun]
+                    [--workload decode|continuous|served|prefix|products|kodisun|surasun]
 
 Random bfloat16 weights, uniform-random prompts of 2,048 tokens, greedy decoding
 through the engine's own step loop (scheduler, step function, sampling). A
@@ -418,6 +418,140 @@ def kodisun(args, sync):
     return 0
 
 
+SURASUN_SHAPES = {
+    # (width, streams, feed-forward inner size, layers as (type, with a feed-forward)); the mixers' sizes follow below
+    "base": (2048, 4, 6144, (("mamba2", False), ("rglru", True), ("parallel", True), ("mamba2", False))),
+    "wide": (4096, 2, 12288, (("rglru", True), ("parallel", True))),
+}
+
+
+def surasun_layers(W, ff, kinds):
+    """Layers of real proportions: Mamba-2 with an inner size of twice the width in heads of 64 and a
+    state of 128; the recurrent unit as wide as the model in blocks of 256; softmax attention in
+    heads of 128, four query heads a key head, beside retention in heads of 128 with values of 256."""
+    mixers = {
+        "mamba2": {"heads": 2 * W // 64, "vdim": 64, "state": 128, "groups": 1, "conv": 4, "norm_groups": 1},
+        "rglru": {"width": W, "blocks": W // 256, "conv": 4},
+        "parallel": {"left": {"heads": W // 128, "kv_heads": W // 512, "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+                              "softcap": 50.0, "rot": {"dims": 64, "base": 10000.0}},
+                     "right": {"heads": W // 256, "dim": 128, "vdim": 256, "rot": {"dims": 128, "base": 10000.0},
+                               "decay": [1.0 - 2.0 ** (-5 - i % 8) for i in range(W // 256)]},
+                     "left_scale": 0.5, "right_scale": 0.5},
+    }
+    return [{"type": kind, "mixer": mixers[kind], "mlp": {"kind": "dense", "ff": ff} if fed else None} for kind, fed in kinds]
+
+
+def surasun(args, sync):
+    """Prefill and decode throughput of the Surasun design at sizes that resemble a real model's
+    layers (random weights, a few layers, a vocabulary of 32,768), beside the Qwen3 dense decoder of
+    the same width and layer count (heads of 128, four query heads a key head, the same feed-forward
+    inner size in every layer). Both go through the engine's own loop: one prompt in one step, then
+    greedy decoding at batch 8 and 64 behind prompts of 1,024 tokens. `frac` prices a prompt's
+    multiply-adds (the products, the recurrences' updates and reads, the attention's pairs) against
+    the bfloat16 matrix peak, and a decode step's bytes (the weights once, the states read and
+    written, the cached keys and values) against the HBM peak."""
+    import torch
+
+    from qwen3_from_scratch_amd.config import ModelConfig
+    from qwen3_from_scratch_amd.config.surasun_config import SurasunConfig
+    from qwen3_from_scratch_amd.engine import SyncEngine, random_model
+
+    vocab, prompt_len, decode_prompt, context = 32768, args.prefill_tokens, 1024, 4096
+    results = {}
+    for shape in ([args.surasun_shape] if args.surasun_shape != "all" else sorted(SURASUN_SHAPES)):
+        W, streams, ff, kinds = SURASUN_SHAPES[shape]
+        if args.layers:
+            kinds = (kinds * args.layers)[:args.layers]
+        listed = surasun_layers(W, ff, kinds)
+        new = SurasunConfig.from_dict({"architecture": "Surasun", "vocab": vocab, "width": W, "norm": {"eps": 1e-5},
+                                       "residual_mult": 1.0, "streams": streams, "layers": listed})
+        dense = ModelConfig.from_dict(dict(QWEN3_8B, vocab_size=vocab, hidden_size=W, num_hidden_layers=len(listed),
+                                           num_attention_heads=W // 128, num_key_value_heads=W // 512, head_dim=128,
+                                           intermediate_size=ff, max_position_embeddings=context))
+        for name, config in (("surasun", new), ("qwen3_dense", dense)):
+            if args.surasun_only and name != args.surasun_only:
+                continue
+            model = random_model(config, dtype=args.dtype, device="cuda:0", seed=0, std=0.02)
+            gen = torch.Generator().manual_seed(1)
+            entry = {}
+            if name == "surasun":
+                matrices = sum(shape_[0] * shape_[1] for key, shape_ in model.tensors().items()
+                               if len(shape_) == 2 and key != "embed" and ".hc" not in key and not key.endswith("conv"))
+                gates = sum(shape_[0] * shape_[1] * shape_[2] for shape_ in model.tensors().values() if len(shape_) == 3)
+                scans = pairs_each = state = cached = 0        # per token: recurrences' multiply-adds; per (query, key) pair; floats of state; cached numbers
+                for layer in listed:
+                    m = layer["mixer"]
+                    if layer["type"] == "mamba2":
+                        scans += 3 * m["heads"] * m["state"] * m["vdim"]
+                        state += m["heads"] * m["state"] * m["vdim"] + 3 * (m["heads"] * m["vdim"] + 2 * m["state"])
+                    elif layer["type"] == "rglru":
+                        state += 4 * m["width"]
+                    else:
+                        scans += 3 * m["right"]["heads"] * m["right"]["dim"] * m["right"]["vdim"]
+                        state += m["right"]["heads"] * m["right"]["dim"] * m["right"]["vdim"]
+                        pairs_each += m["left"]["heads"] * (m["left"]["dim"] + m["left"]["vdim"])
+                        cached += m["left"]["kv_heads"] * (m["left"]["dim"] + m["left"]["vdim"])
+            if "prefill" in args.phases:
+                room = prompt_len + 64
+                engine = SyncEngine(model=model, path="", dtype=args.dtype, device="cuda:0", max_len=room, block_size=BLOCK,
+                                    num_blocks=-(-room // BLOCK), max_num_seqs=1, max_num_tokens=prompt_len,
+                                    chunked_prefill_size=prompt_len, enable_prefix_cache=False)
+                timings = []
+                for _ in range(4):
+                    engine.add_request(torch.randint(0, vocab, (prompt_len,), generator=gen).tolist(),
+                                       engine.default_params(1, temperature=0.0, ignore_eos=True))
+                    sync()
+                    t0 = time.perf_counter()
+                    engine.step()
+                    sync()
+                    timings.append(time.perf_counter() - t0)
+                    while engine.scheduler.has_work():
+                        engine.step()
+                seconds = sorted(timings[1:])[1]
+                if name == "surasun":
+                    flops = (2.0 * prompt_len * (matrices + gates + scans) + 2.0 * vocab * W
+                             + 2.0 * (prompt_len * (prompt_len + 1) / 2) * pairs_each)
+                else:
+                    flops = prefill_flops(config, prompt_len)
+                entry["prefill"] = {"tokens": prompt_len, "tokens_per_s": round(prompt_len / seconds, 1),
+                                    "ms": round(seconds * 1e3, 3), "frac": round(flops / seconds / PEAK_FLOPS[args.dtype], 4)}
+                del engine
+            for batch in ((8, 64) if "decode" in args.phases else ()):
+                engine = SyncEngine(model=model, path="", dtype=args.dtype, device="cuda:0", max_len=context,
+                                    block_size=BLOCK, num_blocks=batch * (context // BLOCK), max_num_seqs=batch,
+                                    max_num_tokens=max(2048, batch), chunked_prefill_size=2048, enable_prefix_cache=False)
+                params = engine.default_params(context - decode_prompt - 1, temperature=0.0, ignore_eos=True)
+                requests = [engine.add_request(torch.randint(0, vocab, (decode_prompt,), generator=gen).tolist(), params)
+                            for _ in range(batch)]
+                while any(r.is_prefill for r in requests) or len(engine.scheduler.waiting):
+                    engine.step()
+                for _ in range(args.warmup):
+                    engine.step()
+                sync()
+                t0 = time.perf_counter()
+                for _ in range(args.steps):
+                    engine.step()
+                sync()
+                step_s = (time.perf_counter() - t0) / args.steps
+                seen = decode_prompt + args.warmup + args.steps // 2
+                if name == "surasun":
+                    need = 2 * (matrices + vocab * W) + 4 * gates + batch * (8 * state + 2 * cached * seen)
+                else:
+                    need = decode_bytes(config, [seen] * batch, 2)
+                entry["decode_b%d" % batch] = {"tokens_per_s": round(batch / step_s, 1), "ms_per_step": round(step_s * 1e3, 3),
+                                               "frac_hbm": round(need / step_s / PEAK_HBM, 4)}
+                del engine
+            results.setdefault(shape, {})[name] = entry
+            del model
+            torch.cuda.empty_cache()
+        results[shape]["sizes"] = {"width": W, "streams": streams, "ff": ff, "layers": [k + ("+ff" if f else "") for k, f in kinds],
+                                   "vocab": vocab}
+    print(json.dumps({"metric": "Surasun beside the Qwen3 dense decoder at equal size: prefill and decode tokens/s",
+                      "unit": "tokens/s", "n_gpus": 1, "higher_is_better": True, "dtype": "bf16", "data": "synthetic",
+                      "steps": args.steps, "warmup": args.warmup, "shapes": results}))
+    return 0
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -429,15 +563,17 @@ def main():
     ap.add_argument("--shape", default="8b", choices=sorted(SHAPES))
     ap.add_argument("--prompt", type=int, default=2048, help="tokens every request holds when decoding starts")
     ap.add_argument("--context", type=int, default=8192, help="tokens of cache per request")
-    ap.add_argument("--workload", default="decode", choices=["decode", "continuous", "served", "prefix", "products", "kodisun"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "continuous", "served", "prefix", "products", "kodisun", "surasun"],
                     help="continuous: 64 requests at once, prompts of 128 to 4,096 tokens, 64 to 512 generated "
                          "tokens each, prompts in portions of 512 (its own JSON line; --steps and --warmup unused); "
                          "prefix: 64 requests that share their first 2,048 tokens, with the prefix index on and off; "
                          "products: a layer's four products by the chosen kernel and by each tile shape of the "
-                         "hand-written one; kodisun: the Kodisun design beside the dense decoder at equal size")
+                         "hand-written one; kodisun, surasun: that design beside the dense decoder at equal size")
     ap.add_argument("--kodisun-shape", default="all", choices=["all"] + sorted(KODISUN_SHAPES))
     ap.add_argument("--kodisun-only", default="", choices=["", "kodisun", "qwen3_dense"], help="one of the two models")
-    ap.add_argument("--phases", default="prefill,decode", help="of --workload kodisun: prefill, decode or both")
+    ap.add_argument("--surasun-shape", default="all", choices=["all"] + sorted(SURASUN_SHAPES))
+    ap.add_argument("--surasun-only", default="", choices=["", "surasun", "qwen3_dense"], help="one of the two models")
+    ap.add_argument("--phases", default="prefill,decode", help="of --workload kodisun or surasun: prefill, decode or both")
     ap.add_argument("--single-copy", action="store_true",
                     help="hold the matrices once (no tile-ordered copy for steps of few rows): half the weights' memory, slower decoding")
     ap.add_argument("--no-points", action="store_true", help="skip the batch-1 and batch-64 points")
@@ -461,6 +597,10 @@ def main():
         torch.cuda.set_device(0)
         args.steps, args.warmup = min(args.steps, 32), min(args.warmup, 8)
         return kodisun(args, torch.cuda.synchronize)
+    if args.workload == "surasun":
+        torch.cuda.set_device(0)
+        args.steps, args.warmup = min(args.steps, 32), min(args.warmup, 8)
+        return surasun(args, torch.cuda.synchronize)
     shape_name, raw = SHAPES[args.shape]
     raw = dict(raw)
     prompt_len, context = args.prompt, args.context

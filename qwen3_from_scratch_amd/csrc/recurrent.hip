@@ -244,6 +244,408 @@ __global__ void retention_scan_kernel(const TA* __restrict__ rows, const float* 
   }
 }
 
+// ---- recurrences with a decayed outer-product state, many tokens at a time ----
+// Mamba-2 and retention are both   S_t = a_t S_(t-1) + k_t v_t^T,   o_t = S_t^T q_t   per head, with
+// a_t = exp(ld_t) <= 1 (retention: a constant per head; Mamba-2: exp(-rate step_t), q = C, k = B,
+// v = step_t x_t). A sequence's rows are cut into chunks of 64. With la_t the sum of ld over the
+// chunk's rows up to and including t, and S the state before the chunk:
+//   o_t = exp(la_t) S^T q_t + sum_{s <= t} exp(la_t - la_s) (q_t . k_s) v_s
+//   S'  = exp(la_last) S + sum_s exp(la_last - la_s) k_s v_s^T
+// Three kernels: every chunk's own sum of outer products (all chunks at once); the states before
+// every chunk, one chunk after the other (a multiply-add per number and chunk); every chunk's
+// results (all chunks at once). Inputs are float32: q and k (T, groups, d), heads_per_group heads
+// share a group's q and k; v (T, H, dv); ld[t * ld_row + h] (ld_row 0: one number per head).
+#define Q3_CHUNK 64
+
+__device__ inline int chunks_before(const int* __restrict__ cu, int b) {
+  int n = 0;
+  for (int i = 0; i < b; ++i) n += (cu[i + 1] - cu[i] + Q3_CHUNK - 1) / Q3_CHUNK;
+  return n;
+}
+
+// la of the chunk's rows into shared memory (one thread; 64 additions), returns nothing.
+__device__ inline void chunk_decays(float* la, const float* __restrict__ ld, long ld_row, int h, int row0, int len) {
+  if (threadIdx.x == 0) {
+    float run = 0.f;
+    for (int s = 0; s < Q3_CHUNK; ++s) {
+      if (s < len) run += ld[(size_t)(row0 + s) * ld_row + h];
+      la[s] = run;
+    }
+  }
+}
+
+// grid (chunks of the longest sequence, H * dv tiles of 64, B); 256 threads. U[i][j] = sum_s
+// exp(la_last - la_s) k_s[i] v_s[j] for the tile's 64 columns j, into `sums` (chunk, H, d, dv);
+// the chunk's whole decay exp(la_last) into `decays` (chunk, H).
+template <int DMAX>
+__global__ void __launch_bounds__(256) chunk_state_kernel(const float* __restrict__ k, const float* __restrict__ v,
+                                                          const float* __restrict__ ld, long ld_row,
+                                                          const int* __restrict__ cu, float* __restrict__ sums,
+                                                          float* __restrict__ decays, int H, int hpg, int d, int dv) {
+  extern __shared__ float lds[];
+  float* kw = lds;                          // (64, d)
+  float* vt = kw + Q3_CHUNK * d;            // (64, 64)
+  __shared__ float la[Q3_CHUNK];
+  const int b = blockIdx.z;
+  const int tiles = (dv + 63) / 64;
+  const int h = blockIdx.y / tiles, tile = blockIdx.y % tiles;
+  const int start = cu[b], n = cu[b + 1] - start;
+  const int c = blockIdx.x;
+  if (c * Q3_CHUNK >= n) return;
+  const int row0 = start + c * Q3_CHUNK;
+  const int len = n - c * Q3_CHUNK < Q3_CHUNK ? n - c * Q3_CHUNK : Q3_CHUNK;
+  const int chunk = chunks_before(cu, b) + c;
+  const int G = H / hpg, g = h / hpg;
+  chunk_decays(la, ld, ld_row, h, row0, len);
+  __syncthreads();
+  const float last = la[len - 1];
+  for (int e = threadIdx.x; e < Q3_CHUNK * d; e += 256) {
+    const int s = e / d, i = e % d;
+    kw[e] = s < len ? k[((size_t)(row0 + s) * G + g) * d + i] * expf(last - la[s]) : 0.f;
+  }
+  for (int e = threadIdx.x; e < Q3_CHUNK * 64; e += 256) {
+    const int s = e / 64, j = tile * 64 + e % 64;
+    vt[e] = (s < len && j < dv) ? v[((size_t)(row0 + s) * H + h) * dv + j] : 0.f;
+  }
+  __syncthreads();
+  const int ti = threadIdx.x / 16, tj = threadIdx.x % 16;
+  float acc[DMAX / 16][4];
+#pragma unroll
+  for (int r = 0; r < DMAX / 16; ++r)
+#pragma unroll
+    for (int x = 0; x < 4; ++x) acc[r][x] = 0.f;
+  for (int s = 0; s < len; ++s) {
+    const float4 vv = *reinterpret_cast<const float4*>(vt + s * 64 + 4 * tj);
+#pragma unroll
+    for (int r = 0; r < DMAX / 16; ++r) {
+      if (ti + 16 * r < d) {
+        const float kv = kw[s * d + ti + 16 * r];
+        acc[r][0] += kv * vv.x;
+        acc[r][1] += kv * vv.y;
+        acc[r][2] += kv * vv.z;
+        acc[r][3] += kv * vv.w;
+      }
+    }
+  }
+  float* dst = sums + ((size_t)chunk * H + h) * d * dv;
+#pragma unroll
+  for (int r = 0; r < DMAX / 16; ++r) {
+    const int i = ti + 16 * r;
+    if (i < d) {
+#pragma unroll
+      for (int x = 0; x < 4; ++x) {
+        const int j = tile * 64 + 4 * tj + x;
+        if (j < dv) dst[(size_t)i * dv + j] = acc[r][x];
+      }
+    }
+  }
+  if (tile == 0 && threadIdx.x == 0) decays[(size_t)chunk * H + h] = expf(last);
+}
+
+// grid (d * dv / 256, H, B): one number of the state per thread, through the sequence's chunks in
+// order. `sums` receives, in place of each chunk's own sum, the state before that chunk; the state
+// tensor receives the state after the last.
+__global__ void chunk_scan_kernel(float* __restrict__ sums, const float* __restrict__ decays, float* __restrict__ state,
+                                  long state_stride, const int* __restrict__ slots, const int* __restrict__ cu, int H,
+                                  int size) {
+  const int e = blockIdx.x * blockDim.x + threadIdx.x;
+  const int h = blockIdx.y, b = blockIdx.z;
+  if (e >= size) return;
+  const int n = cu[b + 1] - cu[b];
+  if (n <= 0) return;
+  const int chunks = (n + Q3_CHUNK - 1) / Q3_CHUNK;
+  const int first = chunks_before(cu, b);
+  float* mine = state + (size_t)slots[b] * state_stride + (size_t)h * size + e;
+  float S = *mine;
+  for (int c = 0; c < chunks; ++c) {
+    float* at = sums + ((size_t)(first + c) * H + h) * size + e;
+    const float own = *at;
+    *at = S;
+    S = decays[(size_t)(first + c) * H + h] * S + own;
+  }
+  *mine = S;
+}
+
+// grid as chunk_state_kernel. A[t][s] = (q_t . k_s) exp(la_t - la_s) for s <= t, over d in slices of
+// 64 through shared memory; then o[t][j] = sum_s A[t][s] v_s[j] + exp(la_t) sum_i q_t[i] S[i][j] with
+// S the state before the chunk (from `sums`), again in slices of 64 over i.
+__global__ void __launch_bounds__(256) chunk_output_kernel(const float* __restrict__ q, const float* __restrict__ k,
+                                                           const float* __restrict__ v, const float* __restrict__ ld,
+                                                           long ld_row, const int* __restrict__ cu,
+                                                           const float* __restrict__ sums, float* __restrict__ out, int H,
+                                                           int hpg, int d, int dv) {
+  __shared__ float A[Q3_CHUNK * Q3_CHUNK];       // (t, s)
+  __shared__ float one[Q3_CHUNK * 65];           // a slice of q, rows padded to 65
+  __shared__ float two[Q3_CHUNK * 65];           // a slice of k (rows padded), then of S or v (rows of 64)
+  __shared__ float la[Q3_CHUNK];
+  const int b = blockIdx.z;
+  const int tiles = (dv + 63) / 64;
+  const int h = blockIdx.y / tiles, tile = blockIdx.y % tiles;
+  const int start = cu[b], n = cu[b + 1] - start;
+  const int c = blockIdx.x;
+  if (c * Q3_CHUNK >= n) return;
+  const int row0 = start + c * Q3_CHUNK;
+  const int len = n - c * Q3_CHUNK < Q3_CHUNK ? n - c * Q3_CHUNK : Q3_CHUNK;
+  const int chunk = chunks_before(cu, b) + c;
+  const int G = H / hpg, g = h / hpg;
+  chunk_decays(la, ld, ld_row, h, row0, len);
+  const int tt = threadIdx.x / 16, tj = threadIdx.x % 16;      // rows tt + 16 r, columns 4 tj .. 4 tj + 3
+  float acc[4][4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r)
+#pragma unroll
+    for (int x = 0; x < 4; ++x) acc[r][x] = 0.f;
+  // A = q k^T, a slice of 64 of d at a time
+  for (int i0 = 0; i0 < d; i0 += 64) {
+    __syncthreads();
+    for (int e = threadIdx.x; e < Q3_CHUNK * 64; e += 256) {
+      const int s = e / 64, i = i0 + e % 64;
+      const bool in = s < len && i < d;
+      one[s * 65 + e % 64] = in ? q[((size_t)(row0 + s) * G + g) * d + i] : 0.f;
+      two[s * 65 + e % 64] = in ? k[((size_t)(row0 + s) * G + g) * d + i] : 0.f;
+    }
+    __syncthreads();
+    for (int i = 0; i < 64; ++i) {
+      float qv[4], kv[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) qv[r] = one[(tt + 16 * r) * 65 + i];
+#pragma unroll
+      for (int x = 0; x < 4; ++x) kv[x] = two[(4 * tj + x) * 65 + i];
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int x = 0; x < 4; ++x) acc[r][x] += qv[r] * kv[x];
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < 4; ++r)
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+      const int t = tt + 16 * r, s = 4 * tj + x;
+      A[t * Q3_CHUNK + s] = (s <= t && t < len) ? acc[r][x] * expf(la[t] - la[s]) : 0.f;
+      acc[r][x] = 0.f;
+    }
+  // the state's share: exp(la_t) q_t S, a slice of 64 of d at a time
+  const float* S = sums + ((size_t)chunk * H + h) * d * dv;
+  for (int i0 = 0; i0 < d; i0 += 64) {
+    __syncthreads();
+    for (int e = threadIdx.x; e < Q3_CHUNK * 64; e += 256) {
+      const int s = e / 64, i = i0 + e % 64;
+      one[s * 65 + e % 64] = (s < len && i < d) ? q[((size_t)(row0 + s) * G + g) * d + i] : 0.f;
+      const int si = i0 + e / 64, j = tile * 64 + e % 64;
+      two[e] = (si < d && j < dv) ? S[(size_t)si * dv + j] : 0.f;
+    }
+    __syncthreads();
+    for (int i = 0; i < 64; ++i) {
+      const float4 sv = *reinterpret_cast<const float4*>(two + i * 64 + 4 * tj);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float qv = one[(tt + 16 * r) * 65 + i];
+        acc[r][0] += qv * sv.x;
+        acc[r][1] += qv * sv.y;
+        acc[r][2] += qv * sv.z;
+        acc[r][3] += qv * sv.w;
+      }
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const float grow = expf(la[tt + 16 * r]);
+#pragma unroll
+    for (int x = 0; x < 4; ++x) acc[r][x] *= grow;
+  }
+  // the chunk's own share: A v
+  __syncthreads();
+  for (int e = threadIdx.x; e < Q3_CHUNK * 64; e += 256) {
+    const int s = e / 64, j = tile * 64 + e % 64;
+    two[e] = (s < len && j < dv) ? v[((size_t)(row0 + s) * H + h) * dv + j] : 0.f;
+  }
+  __syncthreads();
+  for (int s = 0; s < len; ++s) {
+    const float4 vv = *reinterpret_cast<const float4*>(two + s * 64 + 4 * tj);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const float a = A[(tt + 16 * r) * Q3_CHUNK + s];
+      acc[r][0] += a * vv.x;
+      acc[r][1] += a * vv.y;
+      acc[r][2] += a * vv.z;
+      acc[r][3] += a * vv.w;
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int t = tt + 16 * r;
+    if (t < len) {
+#pragma unroll
+      for (int x = 0; x < 4; ++x) {
+        const int j = tile * 64 + 4 * tj + x;
+        if (j < dv) out[((size_t)(row0 + t) * H + h) * dv + j] = acc[r][x];
+      }
+    }
+  }
+}
+
+// What the three kernels need of Mamba-2's rows: step = softplus(dt + dt_bias); ld = -exp(A_log) step;
+// v = step x; q = C, k = B as float32.
+template <typename TA>
+__global__ void mamba2_prepare_kernel(const TA* __restrict__ xbc, const TA* __restrict__ dt, long dt_stride,
+                                      const float* __restrict__ dt_bias, const float* __restrict__ a_log,
+                                      float* __restrict__ qf, float* __restrict__ kf, float* __restrict__ vf,
+                                      float* __restrict__ ld, int H, int P, int N, int G) {
+  const int t = blockIdx.x;
+  const int C = H * P + 2 * G * N;
+  const TA* row = xbc + (size_t)t * C;
+  for (int e = threadIdx.x; e < H * P; e += blockDim.x) {
+    const int h = e / P;
+    const float step = softplus_value(to_float(dt[(size_t)t * dt_stride + h]) + dt_bias[h]);
+    vf[(size_t)t * H * P + e] = step * to_float(row[e]);
+    if (e % P == 0) ld[(size_t)t * H + h] = -expf(a_log[h]) * step;
+  }
+  for (int e = threadIdx.x; e < G * N; e += blockDim.x) {
+    kf[(size_t)t * G * N + e] = to_float(row[H * P + e]);
+    qf[(size_t)t * G * N + e] = to_float(row[H * P + G * N + e]);
+  }
+}
+
+// y += D x after the three kernels.
+template <typename TA>
+__global__ void mamba2_skip_kernel(const TA* __restrict__ xbc, const float* __restrict__ d_skip, float* __restrict__ y,
+                                   int H, int P, int C) {
+  const int t = blockIdx.x;
+  for (int e = threadIdx.x; e < H * P; e += blockDim.x)
+    y[(size_t)t * H * P + e] += d_skip[e / P] * to_float(xbc[(size_t)t * C + e]);
+}
+
+// Retention's rows for the three kernels: q and k turned by the position (k times k_scale), v as float32.
+template <typename TA>
+__global__ void retention_prepare_kernel(const TA* __restrict__ rows, const float* __restrict__ inv_freq, int half,
+                                         const int* __restrict__ positions, float k_scale, float* __restrict__ qf,
+                                         float* __restrict__ kf, float* __restrict__ vf, int H, int dim, int vdim) {
+  const int t = blockIdx.x;
+  const int hd = H * dim, hv = H * vdim;
+  const TA* row = rows + (size_t)t * (2 * (size_t)hd + 2 * (size_t)hv);
+  const float pos = (float)positions[t];
+  for (int e = threadIdx.x; e < hd; e += blockDim.x) {
+    const int j = e % dim;
+    float qv = to_float(row[e]), kv = to_float(row[hd + e]);
+    if (j < 2 * half) {
+      const bool first = j < half;
+      const int partner = first ? e + half : e - half;
+      const float angle = pos * inv_freq[first ? j : j - half];
+      const float c = cosf(angle), s = sinf(angle);
+      const float qp = to_float(row[partner]), kp = to_float(row[hd + partner]);
+      qv = first ? qv * c - qp * s : qv * c + qp * s;
+      kv = first ? kv * c - kp * s : kv * c + kp * s;
+    }
+    qf[(size_t)t * hd + e] = qv;
+    kf[(size_t)t * hd + e] = kv * k_scale;
+  }
+  for (int e = threadIdx.x; e < hv; e += blockDim.x) vf[(size_t)t * hv + e] = to_float(row[2 * hd + e]);
+}
+
+// One block per (token, head): o divided by its root mean square over the head's vdim numbers, times silu(g).
+template <typename TA>
+__global__ void retention_finish_kernel(const float* __restrict__ o, const TA* __restrict__ rows, float eps,
+                                        TA* __restrict__ out, int H, int dim, int vdim) {
+  __shared__ float scratch[17];
+  const int t = blockIdx.x, h = blockIdx.y;
+  const int hd = H * dim, hv = H * vdim;
+  const float* src = o + ((size_t)t * H + h) * vdim;
+  const TA* gate = rows + (size_t)t * (2 * (size_t)hd + 2 * (size_t)hv) + 2 * hd + hv + h * vdim;
+  float sq = 0.f;
+  for (int j = threadIdx.x; j < vdim; j += blockDim.x) sq += src[j] * src[j];
+  const float inv = rsqrtf(block_sum(sq, scratch) / (float)vdim + eps);
+  for (int j = threadIdx.x; j < vdim; j += blockDim.x)
+    out[(size_t)t * hv + h * vdim + j] = from_float<TA>(src[j] * inv * silu_value(to_float(gate[j])));
+}
+
+// Floats of workspace for a step of T rows in B sequences: q, k, v, ld, the chunks' sums and decays.
+extern "C" long q3_chunked_workspace(int T, int B, int H, int G, int d, int dv) {
+  const long chunks = T / Q3_CHUNK + B;
+  return 2L * T * G * d + (long)T * H * dv + (long)T * H + chunks * H * ((long)d * dv + 1);
+}
+
+static int launch_chunks(const float* qf, const float* kf, const float* vf, const float* ld, long ld_row, float* sums,
+                         float* decays, float* state, long state_stride, const int* slots, const int* cu, float* out,
+                         int B, int max_q_len, int H, int hpg, int d, int dv, hipStream_t stream) {
+  const int chunks = (max_q_len + Q3_CHUNK - 1) / Q3_CHUNK;
+  const int tiles = (dv + 63) / 64;
+  const dim3 grid(chunks, H * tiles, B);
+  const size_t lds = (size_t)(Q3_CHUNK * d + Q3_CHUNK * 64) * sizeof(float);
+#define Q3_STATE(DMAX)                                                                                           \
+  hipLaunchKernelGGL(chunk_state_kernel<DMAX>, grid, dim3(256), lds, stream, kf, vf, ld, ld_row, cu, sums, decays, H, \
+                     hpg, d, dv)
+  if (d <= 64) Q3_STATE(64);
+  else if (d <= 128) Q3_STATE(128);
+  else {
+    // 64 rows of more than 128 numbers and the values' tile pass the 64 KB a launch may ask for unasked
+    const hipError_t allowed = hipFuncSetAttribute(reinterpret_cast<const void*>(chunk_state_kernel<256>),
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (allowed != hipSuccess) return (int)allowed;
+    Q3_STATE(256);
+  }
+#undef Q3_STATE
+  hipLaunchKernelGGL(chunk_scan_kernel, dim3((d * dv + 255) / 256, H, B), dim3(256), 0, stream, sums, decays, state,
+                     state_stride, slots, cu, H, d * dv);
+  hipLaunchKernelGGL(chunk_output_kernel, grid, dim3(256), 0, stream, qf, kf, vf, ld, ld_row, cu, sums, out, H, hpg, d,
+                     dv);
+  return q3_launch_status();
+}
+
+extern "C" int q3_mamba2_chunked(const void* xbc, const void* dt, long dt_stride, const float* dt_bias,
+                                 const float* a_log, const float* d_skip, float* state, long state_stride,
+                                 const int* slots, const int* cu, float* y, float* workspace, int T, int B,
+                                 int max_q_len, int H, int P, int N, int G, int act_dtype, hipStream_t stream) {
+  if (T <= 0 || B <= 0 || H <= 0 || P <= 0 || N <= 0 || G <= 0 || H % G || max_q_len <= 0 || B > 65535)
+    return Q3_ERR_BAD_ARGUMENT;
+  if (N > 256 || (long)H * ((P + 63) / 64) > 65535) return Q3_ERR_UNSUPPORTED;
+  float* qf = workspace;
+  float* kf = qf + (size_t)T * G * N;
+  float* vf = kf + (size_t)T * G * N;
+  float* ld = vf + (size_t)T * H * P;
+  float* sums = ld + (size_t)T * H;
+  float* decays = sums + (size_t)(T / Q3_CHUNK + B) * H * N * P;
+  Q3_DISPATCH_DTYPE(act_dtype, TA,
+                    hipLaunchKernelGGL(mamba2_prepare_kernel<TA>, dim3(T), dim3(256), 0, stream, (const TA*)xbc,
+                                       (const TA*)dt, dt_stride, dt_bias, a_log, qf, kf, vf, ld, H, P, N, G));
+  const int status = launch_chunks(qf, kf, vf, ld, H, sums, decays, state, state_stride, slots, cu, y, B, max_q_len, H,
+                                   H / G, N, P, stream);
+  if (status) return status;
+  Q3_DISPATCH_DTYPE(act_dtype, TA,
+                    hipLaunchKernelGGL(mamba2_skip_kernel<TA>, dim3(T), dim3(256), 0, stream, (const TA*)xbc, d_skip, y,
+                                       H, P, H * P + 2 * G * N));
+  return q3_launch_status();
+}
+
+extern "C" int q3_retention_chunked(const void* rows, const float* inv_freq, int half, const int* positions,
+                                    const float* log_decays, float k_scale, float eps, float* state, long state_stride,
+                                    const int* slots, const int* cu, void* out, float* workspace, float* scratch_out,
+                                    int T, int B, int max_q_len, int H, int dim, int vdim, int act_dtype,
+                                    hipStream_t stream) {
+  if (T <= 0 || B <= 0 || H <= 0 || dim <= 0 || vdim <= 0 || half < 0 || 2 * half > dim || max_q_len <= 0 || B > 65535 ||
+      H > 65535)
+    return Q3_ERR_BAD_ARGUMENT;
+  if (half > 0 && !inv_freq) return Q3_ERR_BAD_ARGUMENT;
+  if (dim > 256 || (long)H * ((vdim + 63) / 64) > 65535) return Q3_ERR_UNSUPPORTED;
+  float* qf = workspace;
+  float* kf = qf + (size_t)T * H * dim;
+  float* vf = kf + (size_t)T * H * dim;
+  float* ld = vf + (size_t)T * H * vdim;          // unused stretch: the decays are one number per head
+  float* sums = ld + (size_t)T * H;
+  float* decays = sums + (size_t)(T / Q3_CHUNK + B) * H * dim * vdim;
+  Q3_DISPATCH_DTYPE(act_dtype, TA,
+                    hipLaunchKernelGGL(retention_prepare_kernel<TA>, dim3(T), dim3(256), 0, stream, (const TA*)rows,
+                                       inv_freq, half, positions, k_scale, qf, kf, vf, H, dim, vdim));
+  const int status = launch_chunks(qf, kf, vf, log_decays, 0, sums, decays, state, state_stride, slots, cu, scratch_out,
+                                   B, max_q_len, H, 1, dim, vdim, stream);
+  if (status) return status;
+  const int threads = vdim >= 256 ? 256 : (vdim >= 128 ? 128 : 64);
+  Q3_DISPATCH_DTYPE(act_dtype, TA,
+                    hipLaunchKernelGGL(retention_finish_kernel<TA>, dim3(T, H), dim3(threads), 0, stream, scratch_out,
+                                       (const TA*)rows, eps, (TA*)out, H, dim, vdim));
+  return q3_launch_status();
+}
+
 // ---- launchers ----
 
 extern "C" int q3_causal_conv(const void* x, long x_stride, const float* in_bias, const float* w, const float* bias,

@@ -672,13 +672,17 @@ def causal_conv(x, weight, bias, state, slots, cu_seqlens_q, seq_index, activati
     return out
 
 
-def mamba2_scan(xbc, dt, dt_bias, a_log, d_skip, state, slots, cu_seqlens_q, heads, vdim, n_state, groups):
+CHUNKED_FROM = 9      # a step whose longest sequence brings this many rows takes the recurrences' chunked kernels
+
+
+def mamba2_scan(xbc, dt, dt_bias, a_log, d_skip, state, slots, cu_seqlens_q, heads, vdim, n_state, groups, max_q_len=1):
     """The Mamba-2 recurrence over a packed step. xbc (T, heads vdim + 2 groups n_state), contiguous,
     rows [x | B | C]; dt (T, heads), rows possibly apart, same dtype; dt_bias, a_log, d_skip float32
     (heads,). Per head h of group g = h // (heads / groups), with step = softplus(dt + dt_bias):
     S <- exp(-exp(a_log) step) S + step B x^T, y = S^T C + d_skip x. state float32 (slots,
     heads n_state vdim) laid out (head, n, column), continued and brought up to date. Returns y
-    float32 (T, heads vdim)."""
+    float32 (T, heads vdim). `max_q_len`: the rows of the step's longest sequence; from `CHUNKED_FROM` on
+    the sequences are worked through in chunks of 64 rows, all chunks at once, instead of row by row."""
     _dev(xbc, dt_bias, a_log, d_skip)
     T = xbc.shape[0]
     _need(xbc.dim() == 2 and xbc.dtype in _DT and xbc.shape[1] == heads * vdim + 2 * groups * n_state,
@@ -690,6 +694,15 @@ def mamba2_scan(xbc, dt, dt_bias, a_log, d_skip, state, slots, cu_seqlens_q, hea
     _need(heads % groups == 0 and n_state <= 256, "groups must divide heads; n_state at most 256")
     B = _sequences(slots, cu_seqlens_q, state, heads * n_state * vdim, "mamba2_scan")
     y = torch.empty((T, heads * vdim), dtype=torch.float32, device=xbc.device)
+    if T and max_q_len >= CHUNKED_FROM:
+        lib = library("recurrent")
+        lib.q3_chunked_workspace.restype = ctypes.c_long
+        work = torch.empty(lib.q3_chunked_workspace(T, B, heads, groups, n_state, vdim), dtype=torch.float32, device=xbc.device)
+        _check(lib.q3_mamba2_chunked(
+            _ptr(xbc), _ptr(dt), ctypes.c_long(stride), _ptr(dt_bias), _ptr(a_log), _ptr(d_skip), _ptr(state),
+            ctypes.c_long(state.stride(0)), _ptr(slots), _ptr(cu_seqlens_q), _ptr(y), _ptr(work), T, B, int(max_q_len),
+            heads, vdim, n_state, groups, _DT[xbc.dtype], _stream()), "mamba2_scan")
+        return y
     if T:
         _check(library("recurrent").q3_mamba2_scan(
             _ptr(xbc), _ptr(dt), ctypes.c_long(stride), _ptr(dt_bias), _ptr(a_log), _ptr(d_skip), _ptr(state),
@@ -758,13 +771,16 @@ def rglru_scan(u, gates, rate, y, y_bias, state, slots, cu_seqlens_q, out_dtype)
     return out
 
 
-def retention_scan(qkvg, heads, dim, vdim, inv_freq, positions, decay, k_scale, eps, state, slots, cu_seqlens_q, out_dtype):
+def retention_scan(qkvg, heads, dim, vdim, inv_freq, positions, decay, k_scale, eps, state, slots, cu_seqlens_q, out_dtype,
+                   max_q_len=1, log_decay=None):
     """Retention over a packed step. qkvg (T, 2 heads dim + 2 heads vdim) contiguous, rows
     [q | k | v | g]. q and k turn by the position over their first 2 len(inv_freq) numbers, pairs
     (i, i + len(inv_freq)), angle = position * inv_freq[i] in float32 (`inv_freq` None: no rotation);
     k is multiplied by `k_scale`. Per head S <- decay S + k v^T, o = S^T q; o is divided by the root
     mean square of the head's vdim numbers (eps inside the root) and multiplied by silu(g). state
-    float32 (slots, heads dim vdim) laid out (head, dim, column). Returns (T, heads vdim)."""
+    float32 (slots, heads dim vdim) laid out (head, dim, column). Returns (T, heads vdim).
+    `max_q_len` as for `mamba2_scan`; the chunked kernels take the decays' logarithms, `log_decay`
+    float32 (heads,), formed here if not given."""
     _dev(qkvg, inv_freq, positions, decay)
     T = qkvg.shape[0]
     _need(qkvg.dim() == 2 and qkvg.dtype in _DT and qkvg.dtype == out_dtype
@@ -778,6 +794,19 @@ def retention_scan(qkvg, heads, dim, vdim, inv_freq, positions, decay, k_scale, 
     _f32(decay, (heads,), "decay")
     B = _sequences(slots, cu_seqlens_q, state, heads * dim * vdim, "retention_scan")
     out = torch.empty((T, heads * vdim), dtype=out_dtype, device=qkvg.device)
+    if T and max_q_len >= CHUNKED_FROM:
+        lib = library("recurrent")
+        lib.q3_chunked_workspace.restype = ctypes.c_long
+        if log_decay is None:
+            log_decay = torch.log(decay.double()).float()
+        _f32(log_decay, (heads,), "log_decay")
+        work = torch.empty(lib.q3_chunked_workspace(T, B, heads, heads, dim, vdim), dtype=torch.float32, device=qkvg.device)
+        raw = torch.empty((T, heads * vdim), dtype=torch.float32, device=qkvg.device)
+        _check(lib.q3_retention_chunked(
+            _ptr(qkvg), _ptr(inv_freq), half, _ptr(positions), _ptr(log_decay), ctypes.c_float(k_scale),
+            ctypes.c_float(eps), _ptr(state), ctypes.c_long(state.stride(0)), _ptr(slots), _ptr(cu_seqlens_q), _ptr(out),
+            _ptr(work), _ptr(raw), T, B, int(max_q_len), heads, dim, vdim, _DT[out_dtype], _stream()), "retention_scan")
+        return out
     if T:
         _check(library("recurrent").q3_retention_scan(
             _ptr(qkvg), _ptr(inv_freq), half, _ptr(positions), _ptr(decay), ctypes.c_float(k_scale), ctypes.c_float(eps),

@@ -70,6 +70,6 @@ class Mamba2(Part):
                               out_dtype=proj.dtype)
         y = ops.mamba2_scan(xbc, proj[:, inner + self.channels:], self.dt_bias, self.a_log, self.skip,
                             cache.state[:, tail:], batch.state_slots, batch.cu_seqlens_q, self.heads, self.vdim,
-                            self.state, self.groups)
+                            self.state, self.groups, max_q_len=batch.max_q_len)
         gated = ops.gated_rmsnorm(y, proj[:, :inner], self.norm, self.norm_groups, self.eps, proj.dtype)
         return self.w_out.forward(gated)

@@ -29,7 +29,7 @@ class Retention(Part):
             raise ValueError("one decay per head: %d for %d heads" % (len(decay), heads))
         self.hidden_size, self.heads, self.dim, self.vdim = hidden_size, heads, dim, vdim
         self.decay_values, self.eps, self.rot_dims, self.rot_base = tuple(decay), float(eps), int(rot_dims), float(rot_base)
-        self.w_in = self.w_out = self.decay = self.inv_freq = None
+        self.w_in = self.w_out = self.decay = self.log_decay = self.inv_freq = None
 
     def cache_need(self):
         return CacheNeed(state_shape=(self.heads * self.dim * self.vdim,), state_dtype=torch.float32)
@@ -44,11 +44,14 @@ class Retention(Part):
         joined = torch.cat([fetch(self._name(n), act, keep=False) for n in ("q", "k", "v", "g")], dim=0)
         self.w_in = LinearWeight(joined.contiguous(), self.precision)
         self.w_out = LinearWeight(fetch(self._name("o"), act), self.precision)
-        self.decay = torch.tensor(self.decay_values, dtype=torch.float64).to(torch.float32).to(self.device)
+        decay = torch.tensor(self.decay_values, dtype=torch.float64)
+        self.decay = decay.to(torch.float32).to(self.device)
+        self.log_decay = torch.log(decay).to(torch.float32).to(self.device)
         self.inv_freq = rotation_frequencies(self.rot_dims, self.rot_base, self.device)
 
     def forward(self, x, batch, cache):
         mixed = ops.retention_scan(self.w_in.forward(x), self.heads, self.dim, self.vdim, self.inv_freq, batch.positions,
                                    self.decay, self.dim ** -0.5, self.eps, cache.state, batch.state_slots,
-                                   batch.cu_seqlens_q, self.precision.act)
+                                   batch.cu_seqlens_q, self.precision.act, max_q_len=batch.max_q_len,
+                                   log_decay=self.log_decay)
         return self.w_out.forward(mixed)

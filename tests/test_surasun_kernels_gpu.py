@@ -86,7 +86,8 @@ def test_causal_conv_continues_its_state(dtype, C, taps, lengths):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("H,P,N,G,lengths", [(4, 32, 32, 1, [6, 1, 3]), (6, 80, 48, 3, [1, 1]), (2, 16, 130, 2, [9])])
+@pytest.mark.parametrize("H,P,N,G,lengths", [(4, 32, 32, 1, [6, 1, 3]), (6, 80, 48, 3, [1, 1]), (2, 16, 130, 2, [9]),
+                                             (4, 64, 128, 2, [130, 1, 64, 65]), (3, 72, 24, 1, [200, 7])])
 def test_mamba2_scan(dtype, H, P, N, G, lengths):
     g = _gen(H * P + N)
     T = sum(lengths)
@@ -94,13 +95,17 @@ def test_mamba2_scan(dtype, H, P, N, G, lengths):
     wide = _rand(g, T, H + 5, dtype=dtype)
     dt = wide[:, 5:]
     dt_bias, a_log, skip = _rand(g, H), _rand(g, H, scale=0.5), _rand(g, H)
-    cu, _, slots = _step(lengths, [1, 3, 0][:len(lengths)])
+    cu, _, slots = _step(lengths, [1, 3, 0, 4][:len(lengths)])
     full = _rand(g, 5, H * N * P + 8, scale=0.3)
     a, b = full.clone(), full.clone()
-    got = ops.mamba2_scan(xbc, dt, dt_bias, a_log, skip, a[:, 8:], slots, cu, H, P, N, G)
+    got = ops.mamba2_scan(xbc, dt, dt_bias, a_log, skip, a[:, 8:], slots, cu, H, P, N, G, max_q_len=max(lengths))
     want = twin.mamba2_scan(xbc, dt, dt_bias, a_log, skip, b[:, 8:], slots, cu, H, P, N, G)
     _close(got, want, 3e-5)
     _close(a, b, 3e-5)
+    if max(lengths) >= ops.CHUNKED_FROM:          # row by row and in chunks: the same results and states
+        c = full.clone()
+        _close(ops.mamba2_scan(xbc, dt, dt_bias, a_log, skip, c[:, 8:], slots, cu, H, P, N, G, max_q_len=1), got, 3e-5)
+        _close(c, a, 3e-5)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -135,7 +140,9 @@ def test_recurrent_unit_gates_and_recurrence(width, blocks, lengths):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("H,dim,vdim,rot,lengths", [(4, 64, 64, 64, [7, 1, 2]), (3, 24, 40, 16, [1, 1]), (2, 136, 200, 0, [5])])
+@pytest.mark.parametrize("H,dim,vdim,rot,lengths", [(4, 64, 64, 64, [7, 1, 2]), (3, 24, 40, 16, [1, 1]), (2, 136, 200, 0, [5]),
+                                                    (2, 128, 256, 128, [130, 1, 64]), (3, 40, 72, 20, [100, 65, 3]),
+                                                    (1, 200, 96, 64, [70])])
 def test_retention_scan(dtype, H, dim, vdim, rot, lengths):
     g = _gen(H * dim + vdim)
     T = sum(lengths)
@@ -147,7 +154,8 @@ def test_retention_scan(dtype, H, dim, vdim, rot, lengths):
     cu, _, slots = _step(lengths, [0, 2, 1][:len(lengths)])
     full = _rand(g, 3, H * dim * vdim + 2, scale=0.2)
     a, b = full.clone(), full.clone()
-    got = ops.retention_scan(rows, H, dim, vdim, inv_freq, positions, decay, dim ** -0.5, 1e-6, a[:, 2:], slots, cu, dtype)
+    got = ops.retention_scan(rows, H, dim, vdim, inv_freq, positions, decay, dim ** -0.5, 1e-6, a[:, 2:], slots, cu, dtype,
+                             max_q_len=max(lengths))
     want = twin.retention_scan(rows, H, dim, vdim, inv_freq, positions, decay, dim ** -0.5, 1e-6, b[:, 2:], slots, cu, dtype)
     _close(got, want, 2e-3 if dtype == torch.float32 else 2e-2)       # the angle at position 100,000 is a float32 product
     _close(a, b, 1e-4)

@@ -343,7 +343,7 @@ def causal_conv(x, weight, bias, state, slots, cu_seqlens_q, seq_index, activati
     return out.to(out_dtype or x.dtype)
 
 
-def mamba2_scan(xbc, dt, dt_bias, a_log, d_skip, state, slots, cu_seqlens_q, heads, vdim, n_state, groups):
+def mamba2_scan(xbc, dt, dt_bias, a_log, d_skip, state, slots, cu_seqlens_q, heads, vdim, n_state, groups, max_q_len=1):
     T = xbc.shape[0]
     inner, gn = heads * vdim, groups * n_state
     x = xbc[:, :inner].float().view(T, heads, vdim)
@@ -413,7 +413,8 @@ def _turn(v, positions, inv_freq, neighbours):
     return out
 
 
-def retention_scan(qkvg, heads, dim, vdim, inv_freq, positions, decay, k_scale, eps, state, slots, cu_seqlens_q, out_dtype):
+def retention_scan(qkvg, heads, dim, vdim, inv_freq, positions, decay, k_scale, eps, state, slots, cu_seqlens_q, out_dtype,
+                   max_q_len=1, log_decay=None):
     T = qkvg.shape[0]
     hd, hv = heads * dim, heads * vdim
     rows = qkvg.float()
