@@ -188,6 +188,36 @@ union Pack16 {
 // normal range, which are zero for our purposes (arguments are <= 0).
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// How a score enters the exponent. Ordinarily as s * scale, counted in units of log 2. A build
+// with Q3_SCORE_CAP (attention_capped.hip) first bends it to cap * tanh(s * scale / cap): the raw
+// score becomes (cap / scale) * tanh(s * scale / cap), so that everything behind it, which
+// multiplies by the scale, goes on as it is. tanh(x) = 1 - 2 / (exp(2 x) + 1) by the hardware's
+// exponential and reciprocal; `in` = 2 log2(e) scale / cap, `out` = cap / scale, `in` 0: no cap.
+#ifdef Q3_SCORE_CAP
+struct ScoreScale {
+  float log2, in, out;
+};
+typedef ScoreScale score_scale_t;
+__device__ __forceinline__ float scale_of(const ScoreScale& s) { return s.log2; }
+__device__ __forceinline__ float capped(float v, const ScoreScale& s) {
+  if (s.in == 0.f) return v;
+  return s.out * (1.f - 2.f * __builtin_amdgcn_rcpf(fast_exp2(v * s.in) + 1.f));
+}
+static float g_score_cap = 0.f;
+extern "C" void q3_set_score_cap(float cap) { g_score_cap = cap; }
+static inline ScoreScale make_score_scale(float scale) {
+  ScoreScale s;
+  s.log2 = scale * 1.4426950408889634f;
+  s.in = g_score_cap > 0.f ? 2.f * 1.4426950408889634f * scale / g_score_cap : 0.f;
+  s.out = g_score_cap > 0.f ? g_score_cap / scale : 0.f;
+  return s;
+}
+#else
+typedef float score_scale_t;
+__device__ __forceinline__ float scale_of(float s) { return s; }
+static inline float make_score_scale(float scale) { return scale * 1.4426950408889634f; }
+#endif
+
 // The softmax update of one block of 16 rows for one 32-key tile. s: this lane's
 // eight raw scores (two key blocks of four). Scores enter scaled by scale_log2
 // only inside the exponent: p = 2^(s * scale - m), with m the running maximum of
@@ -196,11 +226,15 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 // operand and rescales the accumulators only if some row's maximum moved.
 template <int NB>
 __device__ __forceinline__ Pack16 softmax_step(const f32x4_t (&s)[2], bool full, int key0, int grp, int row_pos,
-                                               int window, float scale_log2, float& m_run, float& l_run,
+                                               int window, score_scale_t scale_log2, float& m_run, float& l_run,
                                                f32x4_t (&acc)[NB]) {
   float v[8];
 #pragma unroll
   for (int j = 0; j < 8; ++j) v[j] = s[j >> 2][j & 3];
+#ifdef Q3_SCORE_CAP
+#pragma unroll
+  for (int j = 0; j < 8; ++j) v[j] = capped(v[j], scale_log2);
+#endif
   if (!full) {
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
@@ -212,13 +246,13 @@ __device__ __forceinline__ Pack16 softmax_step(const f32x4_t (&s)[2], bool full,
   }
   float mx = fmaxf(fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3])), fmaxf(fmaxf(v[4], v[5]), fmaxf(v[6], v[7])));
   mx = quad_rows_max(mx);
-  const float m_new = fmaxf(m_run, mx * scale_log2);
+  const float m_new = fmaxf(m_run, mx * scale_of(scale_log2));
   Pack16 p;
   float sum = 0.f;
   if (m_new > -INFINITY) {
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-      const float e = fast_exp2(fmaf(v[j], scale_log2, -m_new));
+      const float e = fast_exp2(fmaf(v[j], scale_of(scale_log2), -m_new));
       sum += e;
       p.e[j] = (__bf16)e;
     }
@@ -342,7 +376,7 @@ __device__ __forceinline__ void load_values(Pack16 (&vt)[D / 16], const TileAddr
 template <int D, int QB>
 __device__ __forceinline__ void attend_tile(const Pack16 (&qreg)[QB][D / 32], const Pack16 (&a)[2][D / 32],
                                             Pack16 (&vt)[D / 16], int key0, int kv_len,
-                                            const int (&row_pos)[QB], int window, float scale_log2,
+                                            const int (&row_pos)[QB], int window, score_scale_t scale_log2,
                                             f32x4_t (&acc)[QB][D / 16], float (&m_run)[QB], float (&l_run)[QB]) {
   const int lane = threadIdx.x & 63;
   const int grp = lane >> 4;
@@ -398,7 +432,7 @@ __device__ __forceinline__ void attend_tiles(const Pack16 (&qreg)[QB][D / 32], P
                                              const bf16_t* __restrict__ v_cache, int num_pages,
                                              const int* __restrict__ bt_row, int Hkv, int g_kv, int page, int first,
                                              int last, int step, int kv_len, const int (&row_pos)[QB], int window,
-                                             float scale_log2, f32x4_t (&acc)[QB][D / 16], float (&m_run)[QB],
+                                             score_scale_t scale_log2, f32x4_t (&acc)[QB][D / 16], float (&m_run)[QB],
                                              float (&l_run)[QB]) {
   if (first >= last) return;
   Pack16 a_nxt[2][D / 32], vt[D / 16];
@@ -430,7 +464,7 @@ __device__ __forceinline__ void attend_tiles_ahead(const Pack16 (&qreg)[QB][D / 
                                                    const bf16_t* __restrict__ v_cache, int num_pages,
                                                    const int* __restrict__ bt_row, int bt_stride, int Hkv, int g_kv,
                                                    int page, int first, int last, int step, int kv_len,
-                                                   const int (&row_pos)[QB], int window, float scale_log2,
+                                                   const int (&row_pos)[QB], int window, score_scale_t scale_log2,
                                                    f32x4_t (&acc)[QB][D / 16], float (&m_run)[QB],
                                                    float (&l_run)[QB]) {
   if (first >= last) return;
@@ -612,7 +646,7 @@ template <int D, bool PREP, typename W, bool AHEAD>
 __global__ __launch_bounds__(256) void attn_decode_kernel(
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, int num_pages, const int* __restrict__ block_table, int bt_stride,
-    const int* __restrict__ cu_q, const int* __restrict__ kv_lens, int Hq, int Hkv, int page, float scale_log2,
+    const int* __restrict__ cu_q, const int* __restrict__ kv_lens, int Hq, int Hkv, int page, score_scale_t scale_log2,
     int window, int splits, float* __restrict__ ws_acc, float* __restrict__ ws_ml, DecodePrep prep) {
   const int b = blockIdx.z, g_kv = blockIdx.y, split = blockIdx.x;
   const int G = Hq / Hkv;
@@ -718,7 +752,7 @@ __global__ __launch_bounds__(256) void attn_decode_kernel(
           for (int j = 0; j < 8; ++j) dot = fmaf((float)qreg[0][i].e[j], sh_k[32 * i + 8 * grp + j], dot);
         dot += __shfl_xor(dot, 16, 64);
         dot += __shfl_xor(dot, 32, 64);
-        if (col < rows) m_new = dot * scale_log2;
+        if (col < rows) m_new = dot * scale_of(scale_log2);
       }
     }
   }
@@ -952,13 +986,17 @@ struct PrefillSmem {
 // softmax_step; the probabilities come back as the P operands of the tile's 32-key halves.
 template <int NB, int KB4>
 __device__ __forceinline__ void softmax_tile(const f32x4_t (&s)[KB4], bool full, int key0, int grp, int row_pos,
-                                             int window, float scale_log2, float& m_run, float& l_run,
+                                             int window, score_scale_t scale_log2, float& m_run, float& l_run,
                                              f32x4_t (&acc)[NB], Pack16 (&p)[KB4 / 2]) {
   constexpr int N = 4 * KB4;
   static_assert(N % 2 == 0, "maxima are taken three at a time");
   float v[N];
 #pragma unroll
   for (int j = 0; j < N; ++j) v[j] = s[j >> 2][j & 3];
+#ifdef Q3_SCORE_CAP
+#pragma unroll
+  for (int j = 0; j < N; ++j) v[j] = capped(v[j], scale_log2);
+#endif
   if (!full) {
     // (the row's position and the lane's first key go through an empty piece of assembly so that the
     // comparisons' operands are worked out here, where they are needed, and not before the branch for
@@ -990,14 +1028,14 @@ __device__ __forceinline__ void softmax_tile(const f32x4_t (&s)[KB4], bool full,
     for (int j = 2; j < N; j += 2) asm("v_max3_f32 %0, %1, %2, %3" : "=v"(mx) : "v"(mx), "v"(v[j]), "v"(v[j + 1]));
   }
   mx = quad_rows_max_of_numbers(mx);
-  const float m_new = max_of_numbers(m_run, mx * scale_log2);
+  const float m_new = max_of_numbers(m_run, mx * scale_of(scale_log2));
   // a row that has seen no key yet has minus infinity here and in all its scores: its terms are
   // exp2(-inf - 0) = 0
   const float m_use = m_new > -INFINITY ? m_new : 0.f;
   float sum = 0.f;
 #pragma unroll
   for (int j = 0; j < N; ++j) {
-    const float e = fast_exp2(fmaf(v[j], scale_log2, -m_use));
+    const float e = fast_exp2(fmaf(v[j], scale_of(scale_log2), -m_use));
     sum += e;
     p[(j >> 2) % (KB4 / 2)].e[4 * ((j >> 2) / (KB4 / 2)) + (j & 3)] = (__bf16)e;  // block kb goes with kb + KB4 / 2
   }
@@ -1016,7 +1054,7 @@ template <int D, int TILE, int STAGES>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_prefill_kernel(
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, const bf16_t* __restrict__ k_cache,
     const bf16_t* __restrict__ v_cache, int num_pages, const int* __restrict__ block_table, int bt_stride,
-    const int* __restrict__ cu_q, const int* __restrict__ kv_lens, int Hq, int Hkv, int page, float scale_log2,
+    const int* __restrict__ cu_q, const int* __restrict__ kv_lens, int Hq, int Hkv, int page, score_scale_t scale_log2,
     int window, int tokens_per_block, int key_splits, float* __restrict__ part_acc, float* __restrict__ part_ml) {
   typedef PrefillSmem<D, TILE> SM;
   constexpr int KB4 = TILE / 16;  // 16-key blocks per tile
@@ -1472,7 +1510,7 @@ static int launch_fast(const void* q, int q_stride, void* out, const void* k_cac
                        int min_q_len, int splits, float* ws_acc, float* ws_ml, int key_splits, float* prompt_ws,
                        hipStream_t stream) {
   const int G = Hq / Hkv;
-  const float scale_log2 = scale * 1.4426950408889634f;
+  const score_scale_t scale_log2 = make_score_scale(scale);
   if (min_q_len * G <= 16) {
     if (window == 0)
       hipLaunchKernelGGL((attn_decode_kernel<D, false, float, true>), dim3(splits, Hkv, B), dim3(256), 0, stream,
@@ -1510,7 +1548,7 @@ static int launch_decode_prep(const void* qkv, void* out, const void* k_cache, c
                               const int* block_table, int bt_stride, const int* cu_q, const int* kv_lens, int B,
                               int Hq, int Hkv, int page, float scale, int window, int splits, float* ws_acc,
                               float* ws_ml, const DecodePrep& prep, hipStream_t stream) {
-  const float scale_log2 = scale * 1.4426950408889634f;
+  const score_scale_t scale_log2 = make_score_scale(scale);
   if (window == 0)
     hipLaunchKernelGGL((attn_decode_kernel<D, true, W, true>), dim3(splits, Hkv, B), dim3(256), 0, stream,
                        (const bf16_t*)qkv, (Hq + 2 * Hkv) * D, (bf16_t*)out, (const bf16_t*)k_cache,
@@ -1577,6 +1615,9 @@ extern "C" int q3_paged_attention(const void* q, int q_stride, void* out, const 
                             T_, Hq, Hkv, page, scale, window, max_q_len, min_q_len, splits, ws_acc, ws_ml,
                             prompt_splits, prompt_workspace, stream);
   }
+#ifdef Q3_SCORE_CAP
+  return Q3_ERR_UNSUPPORTED;      // the capped build has the matrix-core kernels only
+#endif
   Q3_DISPATCH_DTYPE(dtype, TT, return launch_general<TT>(q, q_stride, out, k_cache, v_cache, num_pages,
                                                         block_table, bt_stride, cu_q, kv_lens, B, Hq, Hkv,
                                                         D, page, scale, window, max_q_len, stream));

@@ -1,6 +1,7 @@
 // Softmax attention with biased projections, a norm over the whole query and key projections,
 // a rotation of neighbouring pairs, capped scores, key and value heads of different sizes and a
-// gate per head, over a paged cache: keys (pages, G, page, dim), values (pages, G, page, vdim).
+// gate per head, over a paged cache: keys (pages, G, page, dim), values (pages, G, page, vdim) or,
+// transposed within the page as the matrix-core kernels read them, (pages, G, vdim, page).
 #include "common.h"
 
 // One block per token. The row is [q: H dim | k: G dim | v: G vdim | ...] float32, `bias` covers
@@ -14,7 +15,7 @@ __global__ void softcap_prepare_kernel(const float* __restrict__ rows, long row_
                                        const float* __restrict__ inv_freq, int half, const int* __restrict__ positions,
                                        const int* __restrict__ seq_index, const int* __restrict__ block_table,
                                        int table_width, TA* __restrict__ k_cache, TA* __restrict__ v_cache, int page,
-                                       TA* __restrict__ q_out, int H, int G, int dim, int vdim) {
+                                       TA* __restrict__ q_out, int H, int G, int dim, int vdim, int v_transposed) {
   __shared__ float scratch[17];
   const int t = blockIdx.x;
   const float* row = rows + (size_t)t * row_stride;
@@ -62,7 +63,9 @@ __global__ void softcap_prepare_kernel(const float* __restrict__ rows, long row_
   }
   for (int j = threadIdx.x; j < nv; j += blockDim.x) {
     const int g = j / vdim, e = j % vdim;
-    v_cache[(((size_t)pg * G + g) * page + off) * vdim + e] = from_float<TA>(row[nq + nk + j] + bias[nq + nk + j]);
+    const size_t at = v_transposed ? (((size_t)pg * G + g) * vdim + e) * page + off
+                                   : (((size_t)pg * G + g) * page + off) * vdim + e;
+    v_cache[at] = from_float<TA>(row[nq + nk + j] + bias[nq + nk + j]);
   }
 }
 
@@ -78,7 +81,7 @@ __global__ void __launch_bounds__(64) softcap_attention_kernel(
     const TA* __restrict__ q, const TA* __restrict__ k_cache, const TA* __restrict__ v_cache,
     const int* __restrict__ block_table, int table_width, const int* __restrict__ seq_index,
     const int* __restrict__ positions, float scale, float cap, int window, const float* __restrict__ gate,
-    long gate_stride, TA* __restrict__ out, int H, int G, int dim, int vdim, int page) {
+    long gate_stride, TA* __restrict__ out, int H, int G, int dim, int vdim, int page, int v_transposed) {
   __shared__ float sq[Q3_CAP_DIM_MOST];
   __shared__ float sp[64];
   const int lane = threadIdx.x;
@@ -120,11 +123,13 @@ __global__ void __launch_bounds__(64) softcap_attention_kernel(
       const float pj = sp[jj];
       const int key = j0 + jj;
       const int pg = table[key / page];
-      const TA* vr = v_cache + (((size_t)(pg < 0 ? 0 : pg) * G + g) * page + key % page) * vdim;
+      const size_t head = (size_t)(pg < 0 ? 0 : pg) * G + g;
+      const TA* vr = v_transposed ? v_cache + head * vdim * page + key % page : v_cache + (head * page + key % page) * vdim;
+      const int apart = v_transposed ? page : 1;
 #pragma unroll
       for (int i = 0; i < Q3_CAP_VSLICES; ++i) {
         const int c = lane + 64 * i;
-        if (c < vdim) acc[i] += pj * to_float(vr[c]);
+        if (c < vdim) acc[i] += pj * to_float(vr[(size_t)c * apart]);
       }
     }
     __syncthreads();
@@ -138,25 +143,44 @@ __global__ void __launch_bounds__(64) softcap_attention_kernel(
   }
 }
 
+// out[t, h, :] *= sigmoid(gate[t, h]) for a result that another kernel has left ungated.
+template <typename TA>
+__global__ void gate_heads_kernel(TA* __restrict__ out, const float* __restrict__ gate, long gate_stride, int H, int vdim) {
+  const int t = blockIdx.x;
+  for (int e = threadIdx.x; e < H * vdim; e += blockDim.x) {
+    const float open = 1.f / (1.f + expf(-gate[(size_t)t * gate_stride + e / vdim]));
+    out[(size_t)t * H * vdim + e] = from_float<TA>(to_float(out[(size_t)t * H * vdim + e]) * open);
+  }
+}
+
+extern "C" int q3_gate_heads(void* out, const float* gate, long gate_stride, int T, int H, int vdim, int act_dtype,
+                             hipStream_t stream) {
+  if (T <= 0 || H <= 0 || vdim <= 0) return Q3_ERR_BAD_ARGUMENT;
+  Q3_DISPATCH_DTYPE(act_dtype, TA, hipLaunchKernelGGL(gate_heads_kernel<TA>, dim3(T), dim3(256), 0, stream, (TA*)out,
+                                                      gate, gate_stride, H, vdim));
+  return q3_launch_status();
+}
+
 extern "C" int q3_softcap_prepare(const float* rows, long row_stride, const float* bias, const float* q_weight,
                                   const float* k_weight, float eps, const float* inv_freq, int half,
                                   const int* positions, const int* seq_index, const int* block_table, int table_width,
                                   void* k_cache, void* v_cache, int page, void* q_out, int T, int H, int G, int dim,
-                                  int vdim, int act_dtype, hipStream_t stream) {
+                                  int vdim, int v_transposed, int act_dtype, hipStream_t stream) {
   if (T <= 0 || H <= 0 || G <= 0 || H % G || dim <= 0 || vdim <= 0 || half < 0 || 2 * half > dim) return Q3_ERR_BAD_ARGUMENT;
   if (half > 0 && !inv_freq) return Q3_ERR_BAD_ARGUMENT;
   if (k_cache && (!v_cache || !block_table || page <= 0 || table_width <= 0)) return Q3_ERR_BAD_ARGUMENT;
   Q3_DISPATCH_DTYPE(act_dtype, TA,
                     hipLaunchKernelGGL(softcap_prepare_kernel<TA>, dim3(T), dim3(256), 0, stream, rows, row_stride, bias,
                                        q_weight, k_weight, eps, inv_freq, half, positions, seq_index, block_table,
-                                       table_width, (TA*)k_cache, (TA*)v_cache, page, (TA*)q_out, H, G, dim, vdim));
+                                       table_width, (TA*)k_cache, (TA*)v_cache, page, (TA*)q_out, H, G, dim, vdim,
+                                       v_transposed));
   return q3_launch_status();
 }
 
 extern "C" int q3_softcap_attention(const void* q, const void* k_cache, const void* v_cache, const int* block_table,
                                     int table_width, const int* seq_index, const int* positions, float scale, float cap,
                                     int window, const float* gate, long gate_stride, void* out, int T, int H, int G,
-                                    int dim, int vdim, int page, int act_dtype, hipStream_t stream) {
+                                    int dim, int vdim, int page, int v_transposed, int act_dtype, hipStream_t stream) {
   if (T <= 0 || H <= 0 || G <= 0 || H % G || dim <= 0 || vdim <= 0 || page <= 0 || table_width <= 0 || window < 0 ||
       H > 65535)
     return Q3_ERR_BAD_ARGUMENT;
@@ -165,6 +189,6 @@ extern "C" int q3_softcap_attention(const void* q, const void* k_cache, const vo
                     hipLaunchKernelGGL(softcap_attention_kernel<TA>, dim3(T, H), dim3(64), 0, stream, (const TA*)q,
                                        (const TA*)k_cache, (const TA*)v_cache, block_table, table_width, seq_index,
                                        positions, scale, cap, window, gate, gate_stride, (TA*)out, H, G, dim, vdim,
-                                       page));
+                                       page, v_transposed));
   return q3_launch_status();
 }

@@ -816,7 +816,7 @@ def retention_scan(qkvg, heads, dim, vdim, inv_freq, positions, decay, k_scale, 
 
 
 def softcap_prepare(rows, bias, heads, kv_heads, dim, vdim, q_weight, k_weight, eps, inv_freq, positions, seq_index,
-                    out_dtype, block_table=None, k_cache=None, v_cache=None):
+                    out_dtype, block_table=None, k_cache=None, v_cache=None, values_transposed=False):
     """Queries, keys and values of a step from the float32 rows of their joint product.
 
     rows float32 (T, n), n >= heads dim + kv_heads dim + kv_heads vdim, laid out [q | k | v | ...];
@@ -824,7 +824,8 @@ def softcap_prepare(rows, bias, heads, kv_heads, dim, vdim, q_weight, k_weight, 
     whole projection and multiplied by `q_weight` (heads dim) and `k_weight` (kv_heads dim); the
     first 2 len(inv_freq) numbers of every head turn in pairs (2i, 2i + 1) by position * inv_freq[i].
     Returns q (T, heads, dim) of `out_dtype`; with a cache, keys (pages, kv_heads, page, dim) and
-    values (pages, kv_heads, page, vdim) receive the tokens at their positions."""
+    values (pages, kv_heads, page, vdim), or (pages, kv_heads, vdim, page) with `values_transposed`,
+    receive the tokens at their positions."""
     _dev(bias, q_weight, k_weight, inv_freq, positions, seq_index, block_table, k_cache, v_cache)
     _need(rows.is_cuda and rows.dim() == 2 and rows.dtype == torch.float32 and rows.stride(1) == 1, "rows must be float32 (T, n)")
     T = rows.shape[0]
@@ -846,32 +847,42 @@ def softcap_prepare(rows, bias, heads, kv_heads, dim, vdim, q_weight, k_weight, 
               "a key cache comes with a value cache and an int32 block table")
         page, width = k_cache.shape[2], block_table.shape[1]
         _need(k_cache.dim() == 4 and k_cache.shape[1:] == (kv_heads, page, dim) and v_cache.dim() == 4
-              and v_cache.shape[1:] == (kv_heads, page, vdim) and k_cache.dtype == out_dtype and v_cache.dtype == out_dtype,
+              and v_cache.shape[1:] == ((kv_heads, vdim, page) if values_transposed else (kv_heads, page, vdim))
+              and k_cache.dtype == out_dtype and v_cache.dtype == out_dtype,
               "keys (pages, kv_heads, page, dim) and values (pages, kv_heads, page, vdim) of out_dtype")
     q = torch.empty((T, heads, dim), dtype=out_dtype, device=rows.device)
     if T:
         _check(library("softcap").q3_softcap_prepare(
             _ptr(rows), ctypes.c_long(rows.stride(0)), _ptr(bias), _ptr(q_weight), _ptr(k_weight), ctypes.c_float(eps),
             _ptr(inv_freq), half, _ptr(positions), _ptr(seq_index), _ptr(block_table), width, _ptr(k_cache), _ptr(v_cache),
-            page, _ptr(q), T, heads, kv_heads, dim, vdim, _DT[out_dtype], _stream()), "softcap_prepare")
+            page, _ptr(q), T, heads, kv_heads, dim, vdim, 1 if values_transposed else 0, _DT[out_dtype], _stream()),
+            "softcap_prepare")
     return q
 
 
 def softcap_attention(q, k_cache, v_cache, block_table, cu_seqlens_q, kv_lens, seq_index, positions, max_q_len,
-                      max_kv_len, scale, softcap, window=0, gate=None):
+                      max_kv_len, scale, softcap, window=0, gate=None, values_transposed=False, min_q_len=1,
+                      max_kv_len_of_many=None):
     """Causal softmax attention over a paged cache whose keys and values differ in size.
 
     q (T, heads, dim); keys (pages, kv_heads, page, dim), values (pages, kv_heads, page, vdim); the
     token at row t of sequence seq_index[t] sits at positions[t] and sees the keys at positions
     j <= positions[t] (with `window` > 0 only the last `window` of them). score = (q . k) scale, then
     softcap * tanh(score / softcap) if softcap > 0; softmax in float32. `gate` float32 (T, heads),
-    rows possibly apart: head h's result is multiplied by sigmoid(gate[t, h]). Returns (T, heads vdim)."""
+    rows possibly apart: head h's result is multiplied by sigmoid(gate[t, h]). Returns (T, heads vdim).
+
+    With `values_transposed` the values are (pages, kv_heads, vdim, page), and bfloat16 with equal key
+    and value sizes of 64 or 128 then runs on the matrix cores, through the kernels of
+    `paged_attention` (`min_q_len` and `max_kv_len_of_many` are theirs); everything else takes a
+    general kernel of one wavefront per (token, head)."""
     _dev(q, k_cache, v_cache, block_table, seq_index, positions)
     _need(q.dim() == 3 and q.dtype in _DT, "q must be (T, heads, dim)")
     T, H, dim = q.shape
-    _need(k_cache.dim() == 4 and v_cache.dim() == 4 and k_cache.shape[3] == dim and k_cache.shape[:3] == v_cache.shape[:3]
+    _need(k_cache.dim() == 4 and v_cache.dim() == 4 and k_cache.shape[3] == dim and k_cache.shape[:2] == v_cache.shape[:2]
           and k_cache.dtype == q.dtype and v_cache.dtype == q.dtype, "keys (pages, G, page, dim), values (pages, G, page, vdim)")
-    G, page, vdim = k_cache.shape[1], k_cache.shape[2], v_cache.shape[3]
+    G, page = k_cache.shape[1], k_cache.shape[2]
+    vdim = v_cache.shape[2] if values_transposed else v_cache.shape[3]
+    _need(v_cache.shape[2:] == ((vdim, page) if values_transposed else (page, vdim)), "keys and values differ in their pages")
     _need(H % G == 0 and dim <= 512 and vdim <= 512, "kv heads divide heads; dim and vdim at most 512")
     _need(block_table.dtype == torch.int32 and block_table.dim() == 2, "block_table must be int32 (B, W)")
     _need(positions.dtype == torch.int32 and positions.shape == (T,) and seq_index.dtype == torch.int32
@@ -881,12 +892,21 @@ def softcap_attention(q, k_cache, v_cache, block_table, cu_seqlens_q, kv_lens, s
     if gate is not None:
         stride = _rows_view(gate, "gate")
         _need(gate.shape == (T, H) and gate.dtype == torch.float32, "gate must be float32 (T, heads)")
+    if T and values_transposed and dim == vdim and q.dtype == torch.bfloat16 \
+            and library("attention").q3_paged_attention_fast_path(H, G, dim, page, _DT[q.dtype]):
+        out = paged_attention(q, H, k_cache, v_cache, block_table, cu_seqlens_q, kv_lens, max_q_len, max_kv_len, scale,
+                              window=window, min_q_len=min_q_len, max_kv_len_of_many=max_kv_len_of_many, softcap=softcap)
+        if gate is not None:
+            _check(library("softcap").q3_gate_heads(_ptr(out), _ptr(gate), ctypes.c_long(stride), T, H, vdim,
+                                                    _DT[q.dtype], _stream()), "gate_heads")
+        return out
     out = torch.empty((T, H * vdim), dtype=q.dtype, device=q.device)
     if T:
         _check(library("softcap").q3_softcap_attention(
             _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(seq_index),
             _ptr(positions), ctypes.c_float(scale), ctypes.c_float(softcap), int(window), _ptr(gate),
-            ctypes.c_long(stride), _ptr(out), T, H, G, dim, vdim, page, _DT[q.dtype], _stream()), "softcap_attention")
+            ctypes.c_long(stride), _ptr(out), T, H, G, dim, vdim, page, 1 if values_transposed else 0, _DT[q.dtype],
+            _stream()), "softcap_attention")
     return out
 
 
@@ -986,8 +1006,10 @@ def qk_norm_rope_store(qkv, num_q_heads, num_kv_heads, head_dim, positions, seq_
 
 
 def paged_attention(q, num_q_heads, k_cache, v_cache, block_table, cu_seqlens_q, kv_lens,
-                    max_q_len, max_kv_len, scale, window=0, out=None, min_q_len=1, max_kv_len_of_many=None):
+                    max_q_len, max_kv_len, scale, window=0, out=None, min_q_len=1, max_kv_len_of_many=None, softcap=0.0):
     """Causal softmax attention of packed query rows over paged keys and values.
+    `softcap` > 0: a score s enters the softmax as softcap * tanh(s * scale / softcap); that form
+    exists for the sizes the matrix cores take (a second build of the same kernels) and no other.
 
     q is (T, Hq, D) seen through a row stride (a view of the qkv buffer is
     fine). Keys are cached as (pages, Hkv, page, D), values as
@@ -1029,7 +1051,12 @@ def paged_attention(q, num_q_heads, k_cache, v_cache, block_table, cu_seqlens_q,
         out = torch.empty((T, Hq * D), dtype=q.dtype, device=q.device)
     _need(out.shape == (T, Hq * D) and out.dtype == q.dtype, "out must be (T, Hq D)")
     if T and B:
-        lib = library("attention")
+        lib = library("attention_capped" if softcap > 0 else "attention")
+        if softcap > 0:
+            _need(lib.q3_paged_attention_fast_path(Hq, Hkv, D, page, _DT[q.dtype]) and q.stride(0) % 8 == 0,
+                  "capped scores need bfloat16, a head size of 64 or 128 and pages of a power of two from 16")
+            lib.q3_set_score_cap.restype = None
+            lib.q3_set_score_cap(ctypes.c_float(softcap))
         splits, workspace, prompt_splits, prompt_workspace = 1, None, 1, None
         if lib.q3_paged_attention_fast_path(Hq, Hkv, D, page, _DT[q.dtype]):
             if min_q_len * (Hq // Hkv) <= 16:

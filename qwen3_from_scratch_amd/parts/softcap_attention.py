@@ -21,7 +21,9 @@ class SoftcapAttention(Part):
     j <= i (the last `window` of them, 0: all); head a's result is multiplied by sigmoid(W_g h)_a
     before the output product. The four products are one and leave float32 rows, so biases and
     norms see unrounded numbers; norms, angles, scores and the softmax are float32. Keys (rotated)
-    and values are paged, a page (kv_heads, page, dim) and (kv_heads, page, vdim)."""
+    and values are paged, a page of keys (kv_heads, page, dim) and a page of values (kv_heads, vdim,
+    page), transposed within the page as the matrix-core attention kernels read them: bfloat16 with
+    equal key and value sizes of 64 or 128 runs on those kernels, everything else on a general one."""
 
     graph_safe = True
 
@@ -37,7 +39,7 @@ class SoftcapAttention(Part):
 
     def cache_need(self):
         return CacheNeed(paged=(PagedTensor("keys", (self.kv_heads, self.dim), token_axis=1),
-                                PagedTensor("values", (self.kv_heads, self.vdim), token_axis=1)), window=self.window)
+                                PagedTensor("values", (self.kv_heads, self.vdim), token_axis=2)), window=self.window)
 
     def tensors(self):
         H, G, d, dv, W = self.heads, self.kv_heads, self.dim, self.vdim, self.hidden_size
@@ -64,8 +66,11 @@ class SoftcapAttention(Part):
         q = ops.softcap_prepare(rows, self.bias, H, G, d, dv, self.q_norm, self.k_norm, self.eps, self.inv_freq,
                                 batch.positions, batch.seq_index, self.precision.act,
                                 block_table=cache.block_table if cache.writes else None,
-                                k_cache=keys if cache.writes else None, v_cache=values if cache.writes else None)
+                                k_cache=keys if cache.writes else None, v_cache=values if cache.writes else None,
+                                values_transposed=True)
         mixed = ops.softcap_attention(q, keys, values, cache.block_table, batch.cu_seqlens_q, batch.kv_lens,
                                       batch.seq_index, batch.positions, batch.max_q_len, batch.max_kv_len, self.scale,
-                                      self.softcap, window=self.window, gate=rows[:, (H + G) * d + G * dv:])
+                                      self.softcap, window=self.window, gate=rows[:, (H + G) * d + G * dv:],
+                                      values_transposed=True, min_q_len=batch.min_q_len,
+                                      max_kv_len_of_many=getattr(batch, "max_kv_len_portions", None))
         return self.w_out.forward(mixed)

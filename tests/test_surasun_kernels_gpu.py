@@ -179,41 +179,56 @@ def _paged(g, lengths_before, lengths, page, G, dim, vdim, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("H,G,dim,vdim,rot,page", [(8, 4, 96, 32, 48, 16), (3, 1, 40, 72, 40, 8), (4, 4, 16, 16, 0, 16)])
-def test_capped_attention_prepares_and_attends(dtype, H, G, dim, vdim, rot, page):
+@pytest.mark.parametrize("transposed", [False, True])
+@pytest.mark.parametrize("H,G,dim,vdim,rot,page", [(8, 4, 96, 32, 48, 16), (3, 1, 40, 72, 40, 8), (4, 4, 16, 16, 0, 16),
+                                                   (8, 2, 128, 128, 64, 16), (4, 4, 64, 64, 64, 32), (6, 2, 64, 64, 0, 16)])
+def test_capped_attention_prepares_and_attends(dtype, H, G, dim, vdim, rot, page, transposed):
+    """Both layouts of the values; with transposed values, bfloat16 and equal sizes of 64 or 128 the
+    matrix-core kernels run (the last three cases), else the general one."""
     g = _gen(H * dim + vdim)
-    before, lengths = [37, 0, 130], [5, 21, 1]
+    before, lengths = [37, 0, 130], [5, 21, 1] if dim != 128 else [5, 150, 1]
     T = sum(lengths)
     keys, values, table, positions, kv_lens = _paged(g, before, lengths, page, G, dim, vdim, dtype)
+    if transposed:
+        values = values.transpose(2, 3).contiguous()
     cu, seq, _ = _step(lengths, [0, 1, 2])
     n = H * dim + G * dim + G * vdim
     rows = _rand(g, T, n + H)
     bias, qw, kw = _rand(g, n), _rand(g, H * dim), _rand(g, G * dim)
     inv_freq = torch.tensor([250000.0 ** (-2.0 * i / rot) for i in range(rot // 2)], dtype=torch.float32, device=DEV) if rot else None
     k1, v1, k2, v2 = keys.clone(), values.clone(), keys.clone(), values.clone()
-    q1 = ops.softcap_prepare(rows, bias, H, G, dim, vdim, qw, kw, 1e-6, inv_freq, positions, seq, dtype, table, k1, v1)
-    q2 = twin.softcap_prepare(rows, bias, H, G, dim, vdim, qw, kw, 1e-6, inv_freq, positions, seq, dtype, table, k2, v2)
+    q1 = ops.softcap_prepare(rows, bias, H, G, dim, vdim, qw, kw, 1e-6, inv_freq, positions, seq, dtype, table, k1, v1,
+                             values_transposed=transposed)
+    q2 = twin.softcap_prepare(rows, bias, H, G, dim, vdim, qw, kw, 1e-6, inv_freq, positions, seq, dtype, table, k2, v2,
+                              values_transposed=transposed)
     _close(q1, q2, _tol(dtype))
     _close(k1, k2, _tol(dtype))
     _close(v1, v2, _tol(dtype))
     gate = rows[:, n:]
     for cap, window in ((0.0, 0), (5.0, 0), (50.0, 20), (2.0, 1)):
         got = ops.softcap_attention(q2, k2, v2, table, cu, kv_lens, seq, positions, max(lengths), int(kv_lens.max()),
-                                    dim ** -0.5, cap, window=window, gate=gate)
+                                    dim ** -0.5, cap, window=window, gate=gate, values_transposed=transposed,
+                                    min_q_len=min(lengths))
         want = twin.softcap_attention(q2, k2, v2, table, cu, kv_lens, seq, positions, max(lengths), int(kv_lens.max()),
-                                      dim ** -0.5, cap, window=window, gate=gate)
+                                      dim ** -0.5, cap, window=window, gate=gate, values_transposed=transposed)
         _close(got, want, _tol(dtype))
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_one_far_key_carries_the_softmax(dtype):
+@pytest.mark.parametrize("dim,vdim,transposed", [(32, 48, False), (64, 64, True)])
+def test_one_far_key_carries_the_softmax(dtype, dim, vdim, transposed):
     """A query that matches one key hundreds of positions back, at a page's first or last place:
     with that key's score standing out the result is that key's value, and a kernel that skipped
-    the key, its page or its tile would return something else."""
+    the key, its page or its tile would return something else. Once through the general kernel,
+    once (bfloat16, equal sizes of 64, transposed values) through the matrix-core ones."""
     g = _gen(5)
     H = G = 2
-    dim, vdim, page, L = 32, 48, 16, 700
+    page, L = 16, 700
     keys, values, table, _, _ = _paged(g, [L - 1], [1], page, G, dim, vdim, dtype)
+    if transposed:
+        values = values.transpose(2, 3).contiguous()
+    value_at = (lambda pg, off: values[pg, :, :, off]) if transposed else (lambda pg, off: values[pg, :, off])
+    kw = dict(values_transposed=transposed)
     q = _rand(g, 1, H, dim, dtype=dtype)
     cu, seq, _ = _step([1], [0])
     positions = torch.tensor([L - 1], dtype=torch.int32, device=DEV)
@@ -223,13 +238,15 @@ def test_one_far_key_carries_the_softmax(dtype):
         pg = int(table[0, far // page])
         for h in range(G):
             k[pg, h, far % page] = (q[0, h].float() * 4.0).to(dtype)
-        got = ops.softcap_attention(q, k, values, table, cu, kv_lens, seq, positions, 1, L, 1.0, 0.0)
-        want = values[pg, :, far % page].float().reshape(1, -1)
+        got = ops.softcap_attention(q, k, values, table, cu, kv_lens, seq, positions, 1, L, 1.0, 0.0, **kw)
+        want = value_at(pg, far % page).float().reshape(1, -1)
         assert float((got.float() - want).abs().max()) < 0.05, far
-        seen = ops.softcap_attention(q, k, values, table, cu, kv_lens, seq, positions, 1, L, 1.0, 0.0, window=L - 1 - far + 1)
+        capped = ops.softcap_attention(q, k, values, table, cu, kv_lens, seq, positions, 1, L, 1.0, 500.0, **kw)
+        assert float((capped.float() - want).abs().max()) < 0.05, far
+        seen = ops.softcap_attention(q, k, values, table, cu, kv_lens, seq, positions, 1, L, 1.0, 0.0, window=L - 1 - far + 1, **kw)
         assert float((seen.float() - want).abs().max()) < 0.05, far
         if far < L - 1:
-            hidden = ops.softcap_attention(q, k, values, table, cu, kv_lens, seq, positions, 1, L, 1.0, 0.0, window=L - 1 - far)
+            hidden = ops.softcap_attention(q, k, values, table, cu, kv_lens, seq, positions, 1, L, 1.0, 0.0, window=L - 1 - far, **kw)
             assert float((hidden.float() - want).abs().max()) > 0.3, far
 
 

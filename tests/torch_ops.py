@@ -434,7 +434,7 @@ def retention_scan(qkvg, heads, dim, vdim, inv_freq, positions, decay, k_scale, 
 
 
 def softcap_prepare(rows, bias, heads, kv_heads, dim, vdim, q_weight, k_weight, eps, inv_freq, positions, seq_index,
-                    out_dtype, block_table=None, k_cache=None, v_cache=None):
+                    out_dtype, block_table=None, k_cache=None, v_cache=None, values_transposed=False):
     T = rows.shape[0]
     nq, nk, nv = heads * dim, kv_heads * dim, kv_heads * vdim
     z = rows[:, :nq + nk + nv].float() + bias.float()
@@ -448,13 +448,19 @@ def softcap_prepare(rows, bias, heads, kv_heads, dim, vdim, q_weight, k_weight, 
         pos = positions.long()
         pages = block_table[seq_index.long(), pos // page].long()
         k_cache[pages, :, pos % page] = k.to(k_cache.dtype)
-        v_cache[pages, :, pos % page] = v.reshape(T, kv_heads, vdim).to(v_cache.dtype)
+        if values_transposed:
+            v_cache[pages, :, :, pos % page] = v.reshape(T, kv_heads, vdim).to(v_cache.dtype)
+        else:
+            v_cache[pages, :, pos % page] = v.reshape(T, kv_heads, vdim).to(v_cache.dtype)
     return q.to(out_dtype).contiguous()
 
 
 def softcap_attention(q, k_cache, v_cache, block_table, cu_seqlens_q, kv_lens, seq_index, positions, max_q_len,
-                      max_kv_len, scale, softcap, window=0, gate=None):
+                      max_kv_len, scale, softcap, window=0, gate=None, values_transposed=False, min_q_len=1,
+                      max_kv_len_of_many=None):
     T, H, dim = q.shape
+    if values_transposed:
+        v_cache = v_cache.transpose(2, 3)
     G, page, vdim = k_cache.shape[1], k_cache.shape[2], v_cache.shape[3]
     res = torch.zeros((T, H, vdim), dtype=torch.float32, device=q.device)
     cu, kvl = cu_seqlens_q.tolist(), kv_lens.tolist()
