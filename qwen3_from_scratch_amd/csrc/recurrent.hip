@@ -646,6 +646,97 @@ extern "C" int q3_retention_chunked(const void* rows, const float* inv_freq, int
   return q3_launch_status();
 }
 
+// The recurrent unit's recurrence over long sequences, in segments of 64 rows: every segment's own
+// product of decays and its state from nothing (all segments at once), the states at the segments'
+// starts one after the other, then every segment again from its true start.
+__device__ inline void rglru_step(float& S, float k, float r, float i, float u) {
+  const float log_a = -k * r;
+  S = expf(log_a) * S + sqrtf(-expm1f(2.f * log_a)) * i * u;
+}
+
+__global__ void rglru_segment_kernel(const float* __restrict__ u, const float* __restrict__ gates,
+                                     const float* __restrict__ rate, const int* __restrict__ cu, float* __restrict__ seg_decay,
+                                     float* __restrict__ seg_state, int T, int width) {
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  const int b = blockIdx.z, seg = blockIdx.x;
+  const int start = cu[b], n = cu[b + 1] - start;
+  if (c >= width || seg * Q3_CHUNK >= n) return;
+  const int first = start + seg * Q3_CHUNK;
+  const int last = first + (n - seg * Q3_CHUNK < Q3_CHUNK ? n - seg * Q3_CHUNK : Q3_CHUNK);
+  const float k = rate[c];
+  float S = 0.f, logs = 0.f;
+  for (int t = first; t < last; ++t) {
+    const size_t at = (size_t)t * width + c;
+    logs += -k * gates[at];
+    rglru_step(S, k, gates[at], gates[(size_t)T * width + at], u[at]);
+  }
+  const size_t to = (size_t)(chunks_before(cu, b) + seg) * width + c;
+  seg_decay[to] = expf(logs);
+  seg_state[to] = S;
+}
+
+__global__ void rglru_carry_kernel(const float* __restrict__ seg_decay, float* __restrict__ seg_state,
+                                   float* __restrict__ state, long state_stride, const int* __restrict__ slots,
+                                   const int* __restrict__ cu, int width) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  const int b = blockIdx.y;
+  const int n = cu[b + 1] - cu[b];
+  if (c >= width || n <= 0) return;
+  const int segments = (n + Q3_CHUNK - 1) / Q3_CHUNK, first = chunks_before(cu, b);
+  float* mine = state + (size_t)slots[b] * state_stride + c;
+  float S = *mine;
+  for (int seg = 0; seg < segments; ++seg) {
+    const size_t at = (size_t)(first + seg) * width + c;
+    const float own = seg_state[at];
+    seg_state[at] = S;
+    S = seg_decay[at] * S + own;
+  }
+  *mine = S;
+}
+
+template <typename TO>
+__global__ void rglru_apply_kernel(const float* __restrict__ u, const float* __restrict__ gates,
+                                   const float* __restrict__ rate, const float* __restrict__ y, long y_stride,
+                                   const float* __restrict__ y_bias, const int* __restrict__ cu,
+                                   const float* __restrict__ seg_state, TO* __restrict__ out, int T, int width) {
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  const int b = blockIdx.z, seg = blockIdx.x;
+  const int start = cu[b], n = cu[b + 1] - start;
+  if (c >= width || seg * Q3_CHUNK >= n) return;
+  const int first = start + seg * Q3_CHUNK;
+  const int last = first + (n - seg * Q3_CHUNK < Q3_CHUNK ? n - seg * Q3_CHUNK : Q3_CHUNK);
+  const float k = rate[c], yb = y_bias[c];
+  float S = seg_state[(size_t)(chunks_before(cu, b) + seg) * width + c];
+  for (int t = first; t < last; ++t) {
+    const size_t at = (size_t)t * width + c;
+    rglru_step(S, k, gates[at], gates[(size_t)T * width + at], u[at]);
+    const float z = y[(size_t)t * y_stride + c] + yb;
+    out[at] = from_float<TO>(S * (0.5f * z * (1.f + tanhf(0.79788456080286536f * (z + 0.044715f * z * z * z)))));
+  }
+}
+
+// workspace: 2 * (T / 64 + B) * width floats
+extern "C" int q3_rglru_chunked(const float* u, const float* gates, const float* rate, const float* y, long y_stride,
+                                const float* y_bias, float* state, long state_stride, const int* slots, const int* cu,
+                                void* out, float* workspace, int T, int B, int max_q_len, int width, int out_dtype,
+                                hipStream_t stream) {
+  if (T <= 0 || B <= 0 || width <= 0 || max_q_len <= 0 || B > 65535) return Q3_ERR_BAD_ARGUMENT;
+  const int threads = width >= 256 ? 256 : 64;
+  const int cols = (width + threads - 1) / threads;
+  if (cols > 65535) return Q3_ERR_UNSUPPORTED;
+  const dim3 grid((max_q_len + Q3_CHUNK - 1) / Q3_CHUNK, cols, B);
+  float* seg_decay = workspace;
+  float* seg_state = workspace + (size_t)(T / Q3_CHUNK + B) * width;
+  hipLaunchKernelGGL(rglru_segment_kernel, grid, dim3(threads), 0, stream, u, gates, rate, cu, seg_decay, seg_state, T,
+                     width);
+  hipLaunchKernelGGL(rglru_carry_kernel, dim3(cols, B), dim3(threads), 0, stream, seg_decay, seg_state, state,
+                     state_stride, slots, cu, width);
+  Q3_DISPATCH_DTYPE(out_dtype, TO,
+                    hipLaunchKernelGGL(rglru_apply_kernel<TO>, grid, dim3(threads), 0, stream, u, gates, rate, y, y_stride,
+                                       y_bias, cu, seg_state, (TO*)out, T, width));
+  return q3_launch_status();
+}
+
 // ---- launchers ----
 
 extern "C" int q3_causal_conv(const void* x, long x_stride, const float* in_bias, const float* w, const float* bias,

@@ -748,11 +748,12 @@ def block_gates(u, weights, biases):
     return out
 
 
-def rglru_scan(u, gates, rate, y, y_bias, state, slots, cu_seqlens_q, out_dtype):
+def rglru_scan(u, gates, rate, y, y_bias, state, slots, cu_seqlens_q, out_dtype, max_q_len=1):
     """The real-gated linear recurrence over a packed step, float32: with r = gates[0], i = gates[1],
     a = exp(-rate r): S <- a S + sqrt(1 - a^2) i u; out = S * gelu_tanh(y + y_bias), rounded once to
     `out_dtype`. u (T, width) and gates (2, T, width) float32 contiguous, y float32 (T, width) with
-    rows possibly apart, rate and y_bias float32 (width,), state float32 (slots, width)."""
+    rows possibly apart, rate and y_bias float32 (width,), state float32 (slots, width). A step whose
+    longest sequence (`max_q_len`) passes 64 rows is worked through in segments of 64 rows at once."""
     _dev(u, gates, rate, y_bias)
     _need(u.dim() == 2 and u.dtype == torch.float32, "u must be float32 (T, width)")
     T, width = u.shape
@@ -763,6 +764,13 @@ def rglru_scan(u, gates, rate, y, y_bias, state, slots, cu_seqlens_q, out_dtype)
     _need(y.shape == (T, width) and y.dtype == torch.float32 and out_dtype in _DT, "y must be float32 (T, width)")
     B = _sequences(slots, cu_seqlens_q, state, width, "rglru_scan")
     out = torch.empty((T, width), dtype=out_dtype, device=u.device)
+    if T and max_q_len > 64:
+        work = torch.empty((2 * (T // 64 + B) * width,), dtype=torch.float32, device=u.device)
+        _check(library("recurrent").q3_rglru_chunked(
+            _ptr(u), _ptr(gates), _ptr(rate), _ptr(y), ctypes.c_long(stride), _ptr(y_bias), _ptr(state),
+            ctypes.c_long(state.stride(0)), _ptr(slots), _ptr(cu_seqlens_q), _ptr(out), _ptr(work), T, B, int(max_q_len),
+            width, _DT[out_dtype], _stream()), "rglru_scan")
+        return out
     if T:
         _check(library("recurrent").q3_rglru_scan(
             _ptr(u), _ptr(gates), _ptr(rate), _ptr(y), ctypes.c_long(stride), _ptr(y_bias), _ptr(state),

@@ -75,5 +75,5 @@ class RecurrentUnit(Part):
                             in_bias=self.bias_x)
         gates = ops.block_gates(u, self.gate_weights, self.gate_biases)
         mixed = ops.rglru_scan(u, gates, self.decay_rate, both[:, :w], self.bias_y, cache.state[:, tail:],
-                               batch.state_slots, batch.cu_seqlens_q, self.precision.act)
+                               batch.state_slots, batch.cu_seqlens_q, self.precision.act, max_q_len=batch.max_q_len)
         return self.w_out.forward(mixed)

@@ -118,7 +118,8 @@ def test_gated_rmsnorm(dtype, n, groups):
            _tol(dtype))
 
 
-@pytest.mark.parametrize("width,blocks,lengths", [(160, 2, [5, 1, 12]), (96, 3, [1, 1, 1]), (520, 1, [19])])
+@pytest.mark.parametrize("width,blocks,lengths", [(160, 2, [5, 1, 12]), (96, 3, [1, 1, 1]), (520, 1, [19]),
+                                                  (320, 2, [200, 1, 65]), (96, 1, [64, 129])])
 def test_recurrent_unit_gates_and_recurrence(width, blocks, lengths):
     g = _gen(width)
     T, bw = sum(lengths), width // blocks
@@ -133,7 +134,7 @@ def test_recurrent_unit_gates_and_recurrence(width, blocks, lengths):
     full = _rand(g, 4, width + 3)
     for dtype in DTYPES:
         a, b = full.clone(), full.clone()
-        got = ops.rglru_scan(u, gates, rate, y, y_bias, a[:, 3:], slots, cu, dtype)
+        got = ops.rglru_scan(u, gates, rate, y, y_bias, a[:, 3:], slots, cu, dtype, max_q_len=max(lengths))
         want = twin.rglru_scan(u, gates, rate, y, y_bias, b[:, 3:], slots, cu, dtype)
         _close(got, want, _tol(dtype))
         _close(a, b, 2e-5)

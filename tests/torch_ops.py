@@ -377,7 +377,7 @@ def block_gates(u, weights, biases):
     return torch.sigmoid(z).reshape(2, T, width)
 
 
-def rglru_scan(u, gates, rate, y, y_bias, state, slots, cu_seqlens_q, out_dtype):
+def rglru_scan(u, gates, rate, y, y_bias, state, slots, cu_seqlens_q, out_dtype, max_q_len=1):
     T, width = u.shape
     a = torch.exp(-rate.float() * gates[0])
     push = torch.sqrt(1.0 - a * a) * gates[1] * u.float()
