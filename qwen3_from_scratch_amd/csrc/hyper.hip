@@ -27,7 +27,7 @@ __global__ void embed_streams_kernel(const int* __restrict__ ids, const T* __res
 //   out = (u - mean u) * rsqrt(mean (u - mean u)^2 + eps) * weight,
 // the mean taken first and the deviations squared afterwards. u stays in shared memory between
 // the passes. Everything is float32; `out` is rounded once.
-template <typename TA>
+template <typename TA, int VEC>
 __global__ void hyper_norm_kernel(float* __restrict__ x, const TA* __restrict__ delta, const float* __restrict__ mix,
                                   const float* __restrict__ write, const float* __restrict__ read,
                                   const float* __restrict__ weight, const int* __restrict__ rows,
@@ -45,32 +45,61 @@ __global__ void hyper_norm_kernel(float* __restrict__ x, const TA* __restrict__ 
   __syncthreads();
   float* xs = x + src * S * W;
   float sum = 0.f;
-  for (int j = threadIdx.x; j < W; j += blockDim.x) {
-    float old[Q3_STREAMS_MOST];
+  // VEC columns a thread and turn (four where the width allows: 16-byte loads and stores of the streams)
+  for (int j = threadIdx.x * VEC; j < W; j += blockDim.x * VEC) {
+    float old[Q3_STREAMS_MOST][VEC];
 #pragma unroll
-    for (int s = 0; s < Q3_STREAMS_MOST; ++s) old[s] = s < S ? xs[(size_t)s * W + j] : 0.f;
-    float u = 0.f;
+    for (int s = 0; s < Q3_STREAMS_MOST; ++s) {
+      if (s < S) {
+        if constexpr (VEC == 4) {
+          const float4 v = *reinterpret_cast<const float4*>(xs + (size_t)s * W + j);
+          old[s][0] = v.x, old[s][1] = v.y, old[s][2] = v.z, old[s][3] = v.w;
+        } else {
+          old[s][0] = xs[(size_t)s * W + j];
+        }
+      }
+    }
+    float u[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) u[e] = 0.f;
     if (delta) {
-      const float d = to_float(delta[src * W + j]);
+      float d[VEC];
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) d[e] = to_float(delta[src * W + j + e]);
 #pragma unroll
       for (int t = 0; t < Q3_STREAMS_MOST; ++t) {
         if (t < S) {
-          float v = 0.f;
+          float v[VEC];
 #pragma unroll
-          for (int s = 0; s < Q3_STREAMS_MOST; ++s)
-            if (s < S) v += s_mix[s * S + t] * old[s];
-          v += s_write[t] * d;
-          if (write_back) xs[(size_t)t * W + j] = v;
-          u += s_read[t] * v;
+          for (int e = 0; e < VEC; ++e) {
+            v[e] = 0.f;
+#pragma unroll
+            for (int s = 0; s < Q3_STREAMS_MOST; ++s)
+              if (s < S) v[e] += s_mix[s * S + t] * old[s][e];
+            v[e] += s_write[t] * d[e];
+            u[e] += s_read[t] * v[e];
+          }
+          if (write_back) {
+            if constexpr (VEC == 4)
+              *reinterpret_cast<float4*>(xs + (size_t)t * W + j) = make_float4(v[0], v[1], v[2], v[3]);
+            else
+              xs[(size_t)t * W + j] = v[0];
+          }
         }
       }
     } else {
 #pragma unroll
       for (int s = 0; s < Q3_STREAMS_MOST; ++s)
-        if (s < S) u += s_read[s] * old[s];
+        if (s < S) {
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) u[e] += s_read[s] * old[s][e];
+        }
     }
-    u_row[j] = u;
-    sum += u;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      u_row[j + e] = u[e];
+      sum += u[e];
+    }
   }
   if (!out) return;
   const float mean = block_sum(sum, scratch) / (float)W;
@@ -134,10 +163,16 @@ extern "C" int q3_hyper_norm(float* x, const void* delta, const float* mix, cons
   if ((size_t)W * sizeof(float) > 60 * 1024) return Q3_ERR_UNSUPPORTED;
   if (delta && (!mix || !write)) return Q3_ERR_BAD_ARGUMENT;
   if (out && !weight) return Q3_ERR_BAD_ARGUMENT;
-  Q3_DISPATCH_DTYPE(act_dtype, TA,
-                    hipLaunchKernelGGL(hyper_norm_kernel<TA>, dim3(n_out), dim3(threads_for(W)), (size_t)W * sizeof(float),
-                                       stream, x, (const TA*)delta, mix, write, read, weight, rows, (TA*)out, S, W, eps,
-                                       write_back));
+  if (W % 4 == 0)
+    Q3_DISPATCH_DTYPE(act_dtype, TA,
+                      hipLaunchKernelGGL((hyper_norm_kernel<TA, 4>), dim3(n_out), dim3(threads_for(W / 2)),
+                                         (size_t)W * sizeof(float), stream, x, (const TA*)delta, mix, write, read, weight,
+                                         rows, (TA*)out, S, W, eps, write_back));
+  else
+    Q3_DISPATCH_DTYPE(act_dtype, TA,
+                      hipLaunchKernelGGL((hyper_norm_kernel<TA, 1>), dim3(n_out), dim3(threads_for(W)),
+                                         (size_t)W * sizeof(float), stream, x, (const TA*)delta, mix, write, read, weight,
+                                         rows, (TA*)out, S, W, eps, write_back));
   return q3_launch_status();
 }
 

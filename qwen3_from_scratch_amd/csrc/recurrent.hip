@@ -18,25 +18,48 @@ __device__ inline float sigmoid_value(float z) { return 1.f / (1.f + expf(-z)); 
 template <typename TI, typename TO>
 __global__ void causal_conv_kernel(const TI* __restrict__ x, long x_stride, const float* __restrict__ in_bias,
                                    const float* __restrict__ w, const float* __restrict__ bias,
-                                   const float* __restrict__ state, long state_stride, const int* __restrict__ slots,
+                                   const float* state, long state_stride, const int* __restrict__ slots,
                                    const int* __restrict__ cu, const int* __restrict__ seq_index, TO* __restrict__ out,
-                                   int C, int taps, int act) {
-  const int t = blockIdx.x;
+                                   int T, int C, int taps, int act, int rows_each, float* new_tail) {
+  // a thread takes one channel of `rows_each` rows in a row: its taps and biases stay in registers.
+  // `new_tail` (the state again, given only when every sequence brings one row): the thread then
+  // also moves its sequence's tail up by that row, which nobody else reads in this step.
   const int c = blockIdx.y * blockDim.x + threadIdx.x;
   if (c >= C) return;
-  const int b = seq_index[t];
-  const int start = cu[b];
-  const float* tail = state + (size_t)slots[b] * state_stride;
   const float add = in_bias ? in_bias[c] : 0.f;
-  float acc = bias[c];
-  for (int j = 0; j < taps; ++j) {
-    const int src = t - j;
-    const float v = src >= start ? to_float(x[(size_t)src * x_stride + c]) + add
-                                 : tail[(size_t)(taps - 1 - (start - src)) * C + c];
-    acc += w[(size_t)c * taps + taps - 1 - j] * v;
+  const float base = bias[c];
+  float tap[Q3_TAPS_MOST];
+#pragma unroll
+  for (int j = 0; j < Q3_TAPS_MOST; ++j) tap[j] = j < taps ? w[(size_t)c * taps + taps - 1 - j] : 0.f;
+  const int t0 = blockIdx.x * rows_each;
+  const int t1 = t0 + rows_each < T ? t0 + rows_each : T;
+  for (int t = t0; t < t1; ++t) {
+    const int b = seq_index[t];
+    const int start = cu[b];
+    const float* tail = state + (size_t)slots[b] * state_stride;
+    float acc = base;
+#pragma unroll
+    for (int j = 0; j < Q3_TAPS_MOST; ++j) {
+      if (j < taps) {
+        const int src = t - j;
+        const float v = src >= start ? to_float(x[(size_t)src * x_stride + c]) + add
+                                     : tail[(size_t)(taps - 1 - (start - src)) * C + c];
+        acc += tap[j] * v;
+      }
+    }
+    if (act == 1) acc = silu_value(acc);
+    out[(size_t)t * C + c] = from_float<TO>(acc);
+    if (new_tail) {
+      float* mine = new_tail + (size_t)slots[b] * state_stride;
+      float keep[Q3_TAPS_MOST];
+#pragma unroll
+      for (int k = 0; k < Q3_TAPS_MOST; ++k)
+        if (k < taps - 1) keep[k] = k + 1 < taps - 1 ? mine[(size_t)(k + 1) * C + c] : to_float(x[(size_t)t * x_stride + c]) + add;
+#pragma unroll
+      for (int k = 0; k < Q3_TAPS_MOST; ++k)
+        if (k < taps - 1) mine[(size_t)k * C + c] = keep[k];
+    }
   }
-  if (act == 1) acc = silu_value(acc);
-  out[(size_t)t * C + c] = from_float<TO>(acc);
 }
 
 // The tail after the step: the last taps - 1 inputs of the sequence, from this step's rows or,
@@ -177,21 +200,22 @@ __global__ void rglru_scan_kernel(const float* __restrict__ u, const float* __re
 }
 
 // ---- retention ----
-// One block per (sequence, head), thread v keeps column v of S (dim x vdim) in registers. Rows of
-// the input are [q: H dim | k: H dim | v: H vdim | g: H vdim]. Per token q and k turn by the
-// position (pairs (i, i + half) of their first 2 * half numbers, angle = position * inv_freq[i]),
-// k times k_scale; S = decay S + k v^T, o = S^T q; o is divided by the root mean square of the
-// head's vdim numbers and multiplied by silu(g).
+// One block per (sequence, head, 256 columns of the head's vdim), thread v keeps column v of S
+// (dim x vdim) in registers. Rows of the input are [q: H dim | k: H dim | v: H vdim | g: H vdim]. Per
+// token q and k turn by the position (pairs (i, i + half) of their first 2 * half numbers, angle =
+// position * inv_freq[i]), k times k_scale; S = decay S + k v^T, o = S^T q, left as float32 in
+// `raw` (T, H vdim): the division by the head's root mean square and the gate follow in
+// retention_finish_kernel.
 template <typename TA, int DMAX>
-__global__ void retention_scan_kernel(const TA* __restrict__ rows, const float* __restrict__ inv_freq, int half,
-                                      const int* __restrict__ positions, const float* __restrict__ decays, float k_scale,
-                                      float eps, float* __restrict__ state, long state_stride,
-                                      const int* __restrict__ slots, const int* __restrict__ cu, TA* __restrict__ out,
-                                      int H, int dim, int vdim) {
+__global__ void __launch_bounds__(256) retention_scan_kernel(
+    const TA* __restrict__ rows, const float* __restrict__ inv_freq, int half, const int* __restrict__ positions,
+    const float* __restrict__ decays, float k_scale, float* __restrict__ state, long state_stride,
+    const int* __restrict__ slots, const int* __restrict__ cu, float* __restrict__ raw, int H, int dim, int vdim) {
   __shared__ float sq[DMAX], sk[DMAX];
-  __shared__ float scratch[17];
-  const int v = threadIdx.x;
-  const int h = blockIdx.x, b = blockIdx.y;
+  const int slices = (vdim + 255) / 256;
+  const int h = blockIdx.x / slices;
+  const int v = (blockIdx.x % slices) * 256 + threadIdx.x;
+  const int b = blockIdx.y;
   const int start = cu[b], end = cu[b + 1];
   if (end <= start) return;
   const bool live = v < vdim;
@@ -207,7 +231,8 @@ __global__ void retention_scan_kernel(const TA* __restrict__ rows, const float* 
     const TA* q = row + h * dim;
     const TA* k = row + hd + h * dim;
     const float pos = (float)positions[t];
-    for (int j = v; j < dim; j += blockDim.x) {
+    __syncthreads();
+    for (int j = threadIdx.x; j < dim; j += 256) {
       float qv = to_float(q[j]), kv = to_float(k[j]);
       if (j < 2 * half) {
         const bool first = j < half;
@@ -231,11 +256,7 @@ __global__ void retention_scan_kernel(const TA* __restrict__ rows, const float* 
         acc += S[n] * sq[n];
       }
     }
-    const float total = block_sum(live ? acc * acc : 0.f, scratch);
-    if (live) {
-      const float g = to_float(row[2 * hd + hv + h * vdim + v]);
-      out[(size_t)t * hv + h * vdim + v] = from_float<TA>(acc * rsqrtf(total / (float)vdim + eps) * silu_value(g));
-    }
+    if (live) raw[(size_t)t * hv + h * vdim + v] = acc;
   }
   if (live) {
 #pragma unroll
@@ -741,18 +762,22 @@ extern "C" int q3_rglru_chunked(const float* u, const float* gates, const float*
 
 extern "C" int q3_causal_conv(const void* x, long x_stride, const float* in_bias, const float* w, const float* bias,
                               float* state, long state_stride, const int* slots, const int* cu, const int* seq_index,
-                              void* out, int T, int B, int C, int taps, int act, int in_dtype, int out_dtype,
-                              hipStream_t stream) {
+                              void* out, int T, int B, int C, int taps, int act, int single_rows, int in_dtype,
+                              int out_dtype, hipStream_t stream) {
   if (T <= 0 || B <= 0 || C <= 0 || taps < 1 || taps > Q3_TAPS_MOST || act < 0 || act > 1) return Q3_ERR_BAD_ARGUMENT;
   const int threads = C >= 256 ? 256 : 64;
   const int chunks = (C + threads - 1) / threads;
   if (chunks > 65535) return Q3_ERR_UNSUPPORTED;
+  // `single_rows`: every sequence brings exactly one row (T == B); the tail then moves in the same kernel
+  const bool fused = single_rows && T == B && taps > 1;
+  const int rows_each = fused ? 1 : (T >= 2048 ? 16 : (T >= 256 ? 4 : 1));
   Q3_DISPATCH_DTYPE(in_dtype, TI, Q3_DISPATCH_DTYPE(out_dtype, TO, {
-                      hipLaunchKernelGGL((causal_conv_kernel<TI, TO>), dim3(T, chunks), dim3(threads), 0, stream,
-                                         (const TI*)x, x_stride, in_bias, w, bias, state, state_stride, slots, cu,
-                                         seq_index, (TO*)out, C, taps, act);
+                      hipLaunchKernelGGL((causal_conv_kernel<TI, TO>), dim3((T + rows_each - 1) / rows_each, chunks),
+                                         dim3(threads), 0, stream, (const TI*)x, x_stride, in_bias, w, bias, state,
+                                         state_stride, slots, cu, seq_index, (TO*)out, T, C, taps, act, rows_each,
+                                         fused ? state : (float*)nullptr);
                     }));
-  if (taps > 1)
+  if (taps > 1 && !fused)
     Q3_DISPATCH_DTYPE(in_dtype, TI,
                       hipLaunchKernelGGL(conv_tail_kernel<TI>, dim3(B, chunks), dim3(threads), 0, stream, (const TI*)x,
                                          x_stride, in_bias, state, state_stride, slots, cu, C, taps));
@@ -812,30 +837,33 @@ extern "C" int q3_rglru_scan(const float* u, const float* gates, const float* ra
 template <typename TA>
 static int launch_retention(const void* rows, const float* inv_freq, int half, const int* positions, const float* decays,
                             float k_scale, float eps, float* state, long state_stride, const int* slots, const int* cu,
-                            void* out, int B, int H, int dim, int vdim, hipStream_t stream) {
-  const dim3 grid(H, B);
-  const dim3 block((vdim + 63) / 64 * 64);
-#define Q3_RETENTION(DMAX)                                                                                          \
-  hipLaunchKernelGGL((retention_scan_kernel<TA, DMAX>), grid, block, 0, stream, (const TA*)rows, inv_freq, half,   \
-                     positions, decays, k_scale, eps, state, state_stride, slots, cu, (TA*)out, H, dim, vdim)
+                            void* out, float* raw, int T, int B, int H, int dim, int vdim, hipStream_t stream) {
+  const dim3 grid(H * ((vdim + 255) / 256), B);
+#define Q3_RETENTION(DMAX)                                                                                            \
+  hipLaunchKernelGGL((retention_scan_kernel<TA, DMAX>), grid, dim3(256), 0, stream, (const TA*)rows, inv_freq, half,  \
+                     positions, decays, k_scale, state, state_stride, slots, cu, raw, H, dim, vdim)
   if (dim <= 32) Q3_RETENTION(32);
   else if (dim <= 64) Q3_RETENTION(64);
   else if (dim <= 128) Q3_RETENTION(128);
   else Q3_RETENTION(256);
 #undef Q3_RETENTION
+  const int threads = vdim >= 256 ? 256 : (vdim >= 128 ? 128 : 64);
+  hipLaunchKernelGGL(retention_finish_kernel<TA>, dim3(T, H), dim3(threads), 0, stream, raw, (const TA*)rows, eps,
+                     (TA*)out, H, dim, vdim);
   return q3_launch_status();
 }
 
+// `raw`: float32 (T, H vdim) of scratch for the results before their norm and gate.
 extern "C" int q3_retention_scan(const void* rows, const float* inv_freq, int half, const int* positions,
                                  const float* decays, float k_scale, float eps, float* state, long state_stride,
-                                 const int* slots, const int* cu, void* out, int B, int H, int dim, int vdim,
-                                 int act_dtype, hipStream_t stream) {
-  if (B <= 0 || H <= 0 || dim <= 0 || vdim <= 0 || half < 0 || 2 * half > dim || H > 65535 || B > 65535)
+                                 const int* slots, const int* cu, void* out, float* raw, int T, int B, int H, int dim,
+                                 int vdim, int act_dtype, hipStream_t stream) {
+  if (T <= 0 || B <= 0 || H <= 0 || dim <= 0 || vdim <= 0 || half < 0 || 2 * half > dim || B > 65535 || !raw)
     return Q3_ERR_BAD_ARGUMENT;
   if (half > 0 && !inv_freq) return Q3_ERR_BAD_ARGUMENT;
-  if (dim > 256 || vdim > 1024) return Q3_ERR_UNSUPPORTED;
+  if (dim > 256 || (long)H * ((vdim + 255) / 256) > 65535) return Q3_ERR_UNSUPPORTED;
   Q3_DISPATCH_DTYPE(act_dtype, TA, return launch_retention<TA>(rows, inv_freq, half, positions, decays, k_scale, eps,
-                                                               state, state_stride, slots, cu, out, B, H, dim, vdim,
-                                                               stream));
+                                                               state, state_stride, slots, cu, out, raw, T, B, H, dim,
+                                                               vdim, stream));
   return 0;
 }

@@ -643,13 +643,15 @@ def hyper_norm(x, weight, eps, out_dtype, read=None, delta=None, mix=None, write
     return out
 
 
-def causal_conv(x, weight, bias, state, slots, cu_seqlens_q, seq_index, activation=None, out_dtype=None, in_bias=None):
+def causal_conv(x, weight, bias, state, slots, cu_seqlens_q, seq_index, activation=None, out_dtype=None, in_bias=None,
+                max_q_len=0):
     """A causal convolution per channel over a packed step, continued from each sequence's state.
 
     x (T, C), rows possibly apart; weight float32 (C, taps), the last tap the current token's; bias
     float32 (C,); `in_bias` float32 (C,) is added to x first. state float32 (slots, (taps - 1) * C):
     a sequence's last taps - 1 inputs, oldest first (zeros for a fresh sequence), brought up to
-    date. `activation`: None or "silu". Returns (T, C) of `out_dtype` (x's by default)."""
+    date. `activation`: None or "silu". Returns (T, C) of `out_dtype` (x's by default). `max_q_len` 1
+    says that every sequence brings one row: output and new tail are then one kernel."""
     stride = _rows_view(x, "x")
     T, C = x.shape
     taps = weight.shape[1] if weight.dim() == 2 else 0
@@ -668,7 +670,8 @@ def causal_conv(x, weight, bias, state, slots, cu_seqlens_q, seq_index, activati
         _check(library("recurrent").q3_causal_conv(
             _ptr(x), ctypes.c_long(stride), _ptr(in_bias), _ptr(weight), _ptr(bias), _ptr(state),
             ctypes.c_long(state.stride(0)), _ptr(slots), _ptr(cu_seqlens_q), _ptr(seq_index), _ptr(out), T, B, C, taps,
-            1 if activation == "silu" else 0, _DT[x.dtype], _DT[out_dtype], _stream()), "causal_conv")
+            1 if activation == "silu" else 0, 1 if (max_q_len == 1 and T == B) else 0, _DT[x.dtype], _DT[out_dtype],
+            _stream()), "causal_conv")
     return out
 
 
@@ -797,7 +800,7 @@ def retention_scan(qkvg, heads, dim, vdim, inv_freq, positions, decay, k_scale, 
     if inv_freq is not None:
         half = inv_freq.shape[0]
         _f32(inv_freq, (half,), "inv_freq")
-    _need(2 * half <= dim and dim <= 256 and vdim <= 1024, "the rotation fits the head; dim at most 256, vdim at most 1024")
+    _need(2 * half <= dim and dim <= 256, "the rotation fits the head; dim at most 256")
     _need(positions.dtype == torch.int32 and positions.shape == (T,), "positions must be int32 (T,)")
     _f32(decay, (heads,), "decay")
     B = _sequences(slots, cu_seqlens_q, state, heads * dim * vdim, "retention_scan")
@@ -816,10 +819,11 @@ def retention_scan(qkvg, heads, dim, vdim, inv_freq, positions, decay, k_scale, 
             _ptr(work), _ptr(raw), T, B, int(max_q_len), heads, dim, vdim, _DT[out_dtype], _stream()), "retention_scan")
         return out
     if T:
+        raw = torch.empty((T, heads * vdim), dtype=torch.float32, device=qkvg.device)
         _check(library("recurrent").q3_retention_scan(
             _ptr(qkvg), _ptr(inv_freq), half, _ptr(positions), _ptr(decay), ctypes.c_float(k_scale), ctypes.c_float(eps),
-            _ptr(state), ctypes.c_long(state.stride(0)), _ptr(slots), _ptr(cu_seqlens_q), _ptr(out), B, heads, dim, vdim,
-            _DT[out_dtype], _stream()), "retention_scan")
+            _ptr(state), ctypes.c_long(state.stride(0)), _ptr(slots), _ptr(cu_seqlens_q), _ptr(out), _ptr(raw), T, B,
+            heads, dim, vdim, _DT[out_dtype], _stream()), "retention_scan")
     return out
 
 

@@ -67,7 +67,7 @@ class Mamba2(Part):
         proj = self.w_in.forward(x)
         xbc = ops.causal_conv(proj[:, inner:inner + self.channels], self.conv, self.conv_bias, cache.state[:, :tail],
                               batch.state_slots, batch.cu_seqlens_q, batch.seq_index, activation="silu",
-                              out_dtype=proj.dtype)
+                              out_dtype=proj.dtype, max_q_len=batch.max_q_len)
         y = ops.mamba2_scan(xbc, proj[:, inner + self.channels:], self.dt_bias, self.a_log, self.skip,
                             cache.state[:, tail:], batch.state_slots, batch.cu_seqlens_q, self.heads, self.vdim,
                             self.state, self.groups, max_q_len=batch.max_q_len)

@@ -72,7 +72,7 @@ class RecurrentUnit(Part):
         both = self.w_in.forward(x, out_dtype=torch.float32)
         u = ops.causal_conv(both[:, w:], self.conv, self.conv_bias, cache.state[:, :tail], batch.state_slots,
                             batch.cu_seqlens_q, batch.seq_index, activation=None, out_dtype=torch.float32,
-                            in_bias=self.bias_x)
+                            in_bias=self.bias_x, max_q_len=batch.max_q_len)
         gates = ops.block_gates(u, self.gate_weights, self.gate_biases)
         mixed = ops.rglru_scan(u, gates, self.decay_rate, both[:, :w], self.bias_y, cache.state[:, tail:],
                                batch.state_slots, batch.cu_seqlens_q, self.precision.act, max_q_len=batch.max_q_len)

@@ -69,7 +69,8 @@ def test_hyper_norm(dtype, S, W):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("C,taps,lengths", [(70, 4, [1, 9, 2, 1]), (300, 3, [5, 1, 1, 40]), (64, 2, [3]), (33, 1, [2, 2])])
+@pytest.mark.parametrize("C,taps,lengths", [(70, 4, [1, 9, 2, 1]), (300, 3, [5, 1, 1, 40]), (64, 2, [3]), (33, 1, [2, 2]),
+                                            (80, 4, [1, 1, 1]), (40, 2, [1]), (96, 3, [300, 1, 20]), (64, 4, [2100, 3])])
 def test_causal_conv_continues_its_state(dtype, C, taps, lengths):
     g = _gen(C + taps)
     wide = _rand(g, sum(lengths), C + 24, dtype=dtype)
@@ -79,7 +80,8 @@ def test_causal_conv_continues_its_state(dtype, C, taps, lengths):
     full = _rand(g, 7, (taps - 1) * C + 10)
     for activation, in_bias, out_dtype in ((None, add, torch.float32), ("silu", None, dtype)):
         a, b = full.clone(), full.clone()
-        got = ops.causal_conv(x, weight, bias, a[:, 3:3 + (taps - 1) * C], slots, cu, seq, activation, out_dtype, in_bias)
+        got = ops.causal_conv(x, weight, bias, a[:, 3:3 + (taps - 1) * C], slots, cu, seq, activation, out_dtype, in_bias,
+                              max_q_len=max(lengths))
         want = twin.causal_conv(x, weight, bias, b[:, 3:3 + (taps - 1) * C], slots, cu, seq, activation, out_dtype, in_bias)
         _close(got, want, _tol(out_dtype))
         _close(a, b, 1e-6)

@@ -322,7 +322,8 @@ def _sequences(cu_seqlens_q, slots):
     return [(cu[b], cu[b + 1], int(slot)) for b, slot in enumerate(slots.tolist())]
 
 
-def causal_conv(x, weight, bias, state, slots, cu_seqlens_q, seq_index, activation=None, out_dtype=None, in_bias=None):
+def causal_conv(x, weight, bias, state, slots, cu_seqlens_q, seq_index, activation=None, out_dtype=None, in_bias=None,
+                max_q_len=0):
     T, C = x.shape
     taps = weight.shape[1]
     out = torch.empty((T, C), dtype=torch.float32, device=x.device)
