@@ -34,15 +34,17 @@ __global__ void hyper_norm_kernel(float* __restrict__ x, const TA* __restrict__ 
                                   TA* __restrict__ out, int S, int W, float eps, int write_back) {
   extern __shared__ float u_row[];
   __shared__ float scratch[17];
-  __shared__ float s_mix[Q3_STREAMS_MOST * Q3_STREAMS_MOST], s_write[Q3_STREAMS_MOST], s_read[Q3_STREAMS_MOST];
   const int r = blockIdx.x;
   const size_t src = rows ? (size_t)rows[r] : (size_t)r;
-  if (threadIdx.x < S * S) s_mix[threadIdx.x] = mix ? mix[threadIdx.x] : 0.f;
-  if (threadIdx.x < S) {
-    s_write[threadIdx.x] = write ? write[threadIdx.x] : 0.f;
-    s_read[threadIdx.x] = read ? read[threadIdx.x] : 1.f;
+  // the tables are the same for every thread: scalar loads, no staging and no barrier before the streams' loads
+  float s_mix[Q3_STREAMS_MOST * Q3_STREAMS_MOST], s_write[Q3_STREAMS_MOST], s_read[Q3_STREAMS_MOST];
+#pragma unroll
+  for (int i = 0; i < Q3_STREAMS_MOST; ++i) {
+    s_write[i] = (write && i < S) ? write[i] : 0.f;
+    s_read[i] = i < S ? (read ? read[i] : 1.f) : 0.f;
+#pragma unroll
+    for (int t = 0; t < Q3_STREAMS_MOST; ++t) s_mix[i * Q3_STREAMS_MOST + t] = (mix && i < S && t < S) ? mix[i * S + t] : 0.f;
   }
-  __syncthreads();
   float* xs = x + src * S * W;
   float sum = 0.f;
   // VEC columns a thread and turn (four where the width allows: 16-byte loads and stores of the streams)
@@ -75,7 +77,7 @@ __global__ void hyper_norm_kernel(float* __restrict__ x, const TA* __restrict__ 
             v[e] = 0.f;
 #pragma unroll
             for (int s = 0; s < Q3_STREAMS_MOST; ++s)
-              if (s < S) v[e] += s_mix[s * S + t] * old[s][e];
+              if (s < S) v[e] += s_mix[s * Q3_STREAMS_MOST + t] * old[s][e];
             v[e] += s_write[t] * d[e];
             u[e] += s_read[t] * v[e];
           }
@@ -165,7 +167,7 @@ extern "C" int q3_hyper_norm(float* x, const void* delta, const float* mix, cons
   if (out && !weight) return Q3_ERR_BAD_ARGUMENT;
   if (W % 4 == 0)
     Q3_DISPATCH_DTYPE(act_dtype, TA,
-                      hipLaunchKernelGGL((hyper_norm_kernel<TA, 4>), dim3(n_out), dim3(threads_for(W / 2)),
+                      hipLaunchKernelGGL((hyper_norm_kernel<TA, 4>), dim3(n_out), dim3(W >= 2048 ? 512 : threads_for(W / 2)),
                                          (size_t)W * sizeof(float), stream, x, (const TA*)delta, mix, write, read, weight,
                                          rows, (TA*)out, S, W, eps, write_back));
   else

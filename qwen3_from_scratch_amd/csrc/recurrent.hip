@@ -170,6 +170,51 @@ __global__ void block_gates_kernel(const float* __restrict__ u, const float* __r
   }
 }
 
+// The same for steps of few rows, where the kernel above leaves most of the chip idle: a block
+// takes 64 outputs of one part and gate for eight tokens, its four quarters of threads each a
+// quarter of the inputs; the quarters' sums meet in shared memory in a fixed order.
+__global__ void __launch_bounds__(256) block_gates_few_kernel(const float* __restrict__ u, const float* __restrict__ w,
+                                                              const float* __restrict__ bias, float* __restrict__ out,
+                                                              int T, int width, int bw, int out_tiles) {
+  extern __shared__ float su[];          // (Q3_GATE_TOKENS, bw), then (4, 64, Q3_GATE_TOKENS) partial sums
+  float* part = su + Q3_GATE_TOKENS * bw;
+  const int t0 = blockIdx.x * Q3_GATE_TOKENS;
+  const int b = blockIdx.y / out_tiles, tile = blockIdx.y % out_tiles, g = blockIdx.z;
+  const int blocks = width / bw;
+  for (int i = threadIdx.x; i < Q3_GATE_TOKENS * bw; i += 256) {
+    const int tt = i / bw, e = i % bw;
+    su[i] = t0 + tt < T ? u[(size_t)(t0 + tt) * width + b * bw + e] : 0.f;
+  }
+  __syncthreads();
+  const int lane = threadIdx.x & 63, quarter = threadIdx.x >> 6;
+  const int o = tile * 64 + lane;
+  const int each = (bw + 3) / 4;
+  const int i0 = quarter * each, i1 = i0 + each < bw ? i0 + each : bw;
+  float acc[Q3_GATE_TOKENS];
+#pragma unroll
+  for (int tt = 0; tt < Q3_GATE_TOKENS; ++tt) acc[tt] = 0.f;
+  if (o < bw) {
+    const float* wb = w + ((size_t)g * blocks + b) * bw * bw + o;
+    for (int i = i0; i < i1; ++i) {
+      const float wv = wb[(size_t)i * bw];
+#pragma unroll
+      for (int tt = 0; tt < Q3_GATE_TOKENS; ++tt) acc[tt] += wv * su[tt * bw + i];
+    }
+  }
+#pragma unroll
+  for (int tt = 0; tt < Q3_GATE_TOKENS; ++tt) part[(quarter * 64 + lane) * Q3_GATE_TOKENS + tt] = acc[tt];
+  __syncthreads();
+  if (quarter == 0 && o < bw) {
+    const float start = bias[((size_t)g * blocks + b) * bw + o];
+#pragma unroll
+    for (int tt = 0; tt < Q3_GATE_TOKENS; ++tt) {
+      float total = start;
+      for (int qtr = 0; qtr < 4; ++qtr) total += part[(qtr * 64 + lane) * Q3_GATE_TOKENS + tt];
+      if (t0 + tt < T) out[((size_t)g * T + t0 + tt) * width + b * bw + o] = sigmoid_value(total);
+    }
+  }
+}
+
 // ---- the recurrent unit's recurrence ----
 // Per (sequence, channel): log a = -rate r, a = exp(log a), S = a S + sqrt(1 - a^2) i u (1 - a^2 as
 // -expm1(2 log a)), out = S * gelu_tanh(y + y_bias). gates = [r | i], each (T, width).
@@ -816,6 +861,14 @@ extern "C" int q3_block_gates(const float* u, const float* w, const float* bias,
   if (T <= 0 || width <= 0 || blocks <= 0 || width % blocks || blocks > 65535) return Q3_ERR_BAD_ARGUMENT;
   const int bw = width / blocks;
   if (bw > 1536) return Q3_ERR_UNSUPPORTED;
+  if (T <= 256) {
+    const int out_tiles = (bw + 63) / 64;
+    if ((long)blocks * out_tiles > 65535) return Q3_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL(block_gates_few_kernel, dim3((T + Q3_GATE_TOKENS - 1) / Q3_GATE_TOKENS, blocks * out_tiles, 2),
+                       dim3(256), (size_t)(Q3_GATE_TOKENS * bw + 4 * 64 * Q3_GATE_TOKENS) * sizeof(float), stream, u, w,
+                       bias, out, T, width, bw, out_tiles);
+    return q3_launch_status();
+  }
   const int threads = bw >= 256 ? 256 : (bw >= 128 ? 128 : 64);
   hipLaunchKernelGGL(block_gates_kernel, dim3((T + Q3_GATE_TOKENS - 1) / Q3_GATE_TOKENS, blocks, 2), dim3(threads),
                      (size_t)Q3_GATE_TOKENS * bw * sizeof(float), stream, u, w, bias, out, T, width, bw);

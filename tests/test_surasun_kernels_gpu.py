@@ -121,7 +121,8 @@ def test_gated_rmsnorm(dtype, n, groups):
 
 
 @pytest.mark.parametrize("width,blocks,lengths", [(160, 2, [5, 1, 12]), (96, 3, [1, 1, 1]), (520, 1, [19]),
-                                                  (320, 2, [200, 1, 65]), (96, 1, [64, 129])])
+                                                  (320, 2, [200, 1, 65]), (96, 1, [64, 129]), (2048, 8, [1] * 9),
+                                                  (70, 1, [3, 300])])
 def test_recurrent_unit_gates_and_recurrence(width, blocks, lengths):
     g = _gen(width)
     T, bw = sum(lengths), width // blocks
@@ -132,8 +133,8 @@ def test_recurrent_unit_gates_and_recurrence(width, blocks, lengths):
     rate = _rand(g, width).abs() + 0.01
     y = _rand(g, T, 2 * width)[:, :width]
     y_bias = _rand(g, width)
-    cu, _, slots = _step(lengths, [2, 0, 1][:len(lengths)])
-    full = _rand(g, 4, width + 3)
+    cu, _, slots = _step(lengths, [2, 0, 1, 3, 4, 5, 6, 7, 8][:len(lengths)])
+    full = _rand(g, 9, width + 3)
     for dtype in DTYPES:
         a, b = full.clone(), full.clone()
         got = ops.rglru_scan(u, gates, rate, y, y_bias, a[:, 3:], slots, cu, dtype, max_q_len=max(lengths))
