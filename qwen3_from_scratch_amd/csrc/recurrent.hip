@@ -195,10 +195,17 @@ __global__ void __launch_bounds__(256) block_gates_few_kernel(const float* __res
   for (int tt = 0; tt < Q3_GATE_TOKENS; ++tt) acc[tt] = 0.f;
   if (o < bw) {
     const float* wb = w + ((size_t)g * blocks + b) * bw * bw + o;
-    for (int i = i0; i < i1; ++i) {
-      const float wv = wb[(size_t)i * bw];
+    // eight weights at a time, all asked for before any is used: the loop is a chain of memory round trips otherwise
+    for (int i = i0; i < i1; i += 8) {
+      float wv[8];
 #pragma unroll
-      for (int tt = 0; tt < Q3_GATE_TOKENS; ++tt) acc[tt] += wv * su[tt * bw + i];
+      for (int j = 0; j < 8; ++j) wv[j] = i + j < i1 ? wb[(size_t)(i + j) * bw] : 0.f;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int at = i + j < i1 ? i + j : i0;
+#pragma unroll
+        for (int tt = 0; tt < Q3_GATE_TOKENS; ++tt) acc[tt] += wv[j] * su[tt * bw + at];
+      }
     }
   }
 #pragma unroll
