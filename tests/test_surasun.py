@@ -82,7 +82,23 @@ ODD = {"architecture": "Surasun", "vocab": 53, "width": 40, "norm": {"eps": 1e-5
            _layer("rglru", _unit(35, 5, 2), ff=18),
            _layer("mamba2", _mamba(3, 5, 7, 3, 5, 5)),
        ]}
-CONFIGS = {"mixed": MIXED, "plain": PLAIN, "wide": WIDE, "odd": ODD}
+# sizes at the kernels' ends: eight streams, eight taps, a state of 256, keys of 256 with values that are no
+# multiple of a wavefront, thirty-two query heads on one key head, blocks and norm parts of one number, equal key and
+# value sizes of 64 (the matrix-core attention kernels in bfloat16) with and without a cap
+EDGES = {"architecture": "Surasun", "vocab": 70, "width": 64, "norm": {"eps": 1e-6}, "residual_mult": 0.25, "streams": 8,
+         "layers": [
+             _layer("mamba2", _mamba(2, 4, 256, 2, 8, 8)),
+             _layer("parallel", _sides(32, 1, 8, 4, 8, 5.0, 1, 256, 300, 256, [0.99]), ff=24),
+             _layer("rglru", _unit(24, 24, 8)),
+             _layer("parallel", _sides(4, 2, 64, 64, 32, 12.0, 2, 8, 2, 4, [0.5, 0.9]), ff=24),
+             _layer("parallel", _sides(2, 1, 64, 64, 64, 0.0, 1, 4, 4, 0, [0.7])),
+             _layer("mamba2", _mamba(1, 70, 3, 1, 2, 1)),
+         ]}
+CONFIGS = {"mixed": MIXED, "plain": PLAIN, "wide": WIDE, "odd": ODD, "edges": EDGES}
+# how the float32 folders are written: large weights and peaked queries; the configuration of the kernels' ends, whose
+# long convolutions and wide states carry float32's own rounding furthest, with weights half as large
+SHARP = {name: dict(peak=3.0) for name in CONFIGS}
+SHARP["edges"] = dict(peak=2.0, std=0.1)
 # one layer of each kind, the mixer alone
 ALONE = {kind: {"architecture": "Surasun", "vocab": 61, "width": 32, "norm": {"eps": 1e-5}, "residual_mult": 0.3,
                 "streams": 3, "layers": [_layer(kind, mixer)]}
@@ -112,7 +128,7 @@ def _write(folder, data, seed=5, peak=None, std=0.2):
 
 @pytest.fixture(scope="module", params=sorted(CONFIGS))
 def folder(request, tmp_path_factory):
-    return _write(tmp_path_factory.mktemp(request.param), CONFIGS[request.param], peak=3.0)
+    return _write(tmp_path_factory.mktemp(request.param), CONFIGS[request.param], **SHARP[request.param])
 
 
 @pytest.fixture(scope="module", params=sorted(CONFIGS))
@@ -122,7 +138,7 @@ def folders(request, tmp_path_factory):
     the places where the engine rounds, already moves a row by a twentieth of its spread or more
     (the recurrences carry it on), so bfloat16 gets weights under which that rounding stays at a
     third of the bound below."""
-    return {"float32": _write(tmp_path_factory.mktemp(request.param), CONFIGS[request.param], peak=3.0),
+    return {"float32": _write(tmp_path_factory.mktemp(request.param), CONFIGS[request.param], **SHARP[request.param]),
             "bfloat16": _write(tmp_path_factory.mktemp(request.param + "_b"), CONFIGS[request.param], std=0.06)}
 
 
@@ -231,7 +247,7 @@ def _streams_behind(folder, tokens, device, dtype):
     return seen
 
 
-@pytest.mark.parametrize("name", ["mixed", "plain", "odd"])
+@pytest.mark.parametrize("name", ["mixed", "plain", "odd", "edges"])
 def test_streams_behind_every_layer_on_the_host(cpu_ops, tmp_path, name):
     """The sum of the streams behind every layer, what the last sublayer still owes them included."""
     folder = _write(tmp_path / "m", CONFIGS[name])
