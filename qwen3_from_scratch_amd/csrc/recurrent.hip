@@ -62,6 +62,170 @@ __global__ void causal_conv_kernel(const TI* __restrict__ x, long x_stride, cons
   }
 }
 
+// Eight channels a thread in 16-byte accesses, for steps of many rows: the thread walks `rows_each`
+// rows with its last taps - 1 inputs in registers, so every input is read once; where a row is a
+// sequence's first (or the thread's first), the inputs before it come from the rows above or from
+// the sequence's tail. Needs C and the rows' stride in steps of eight and 16-byte aligned rows.
+__device__ inline void load8(const bf16_t* p, float (&v)[8]) {
+  union {
+    uint4 u;
+    bf16_t e[8];
+  } a;
+  a.u = *reinterpret_cast<const uint4*>(p);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) v[i] = bf16_to_float(a.e[i]);
+}
+__device__ inline void load8(const float* p, float (&v)[8]) {
+  const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+  v[0] = a.x, v[1] = a.y, v[2] = a.z, v[3] = a.w, v[4] = b.x, v[5] = b.y, v[6] = b.z, v[7] = b.w;
+}
+__device__ inline void store8(bf16_t* p, const float (&v)[8]) {
+  union {
+    uint4 u;
+    bf16_t e[8];
+  } a;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) a.e[i] = float_to_bf16(v[i]);
+  *reinterpret_cast<uint4*>(p) = a.u;
+}
+__device__ inline void store8(float* p, const float (&v)[8]) {
+  *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+  *reinterpret_cast<float4*>(p + 4) = make_float4(v[4], v[5], v[6], v[7]);
+}
+
+#define Q3_CONV_TILE 8
+template <typename TI, typename TO>
+__global__ void __launch_bounds__(64) causal_conv_wide_kernel(const TI* __restrict__ x, long x_stride, const float* __restrict__ in_bias,
+                                        const float* __restrict__ w, const float* __restrict__ bias,
+                                        const float* __restrict__ state, long state_stride,
+                                        const int* __restrict__ slots, const int* __restrict__ cu,
+                                        const int* __restrict__ seq_index, TO* __restrict__ out, int T, int C, int taps,
+                                        int act, int rows_each) {
+  // the block's taps lie side by side in memory (64 threads x 8 channels x taps): in through shared memory
+  __shared__ __attribute__((aligned(16))) float taps_of_block[64 * 8 * Q3_TAPS_MOST];
+  const int first = blockIdx.y * 64 * 8;
+  const int held = C - first < 64 * 8 ? C - first : 64 * 8;
+  {
+    // 2 * taps loads of 16 bytes a thread, all asked for before the first is stored
+    const float4* src = reinterpret_cast<const float4*>(w + (size_t)first * taps);
+    const int pieces = held * taps / 4;
+    float4 got[2 * Q3_TAPS_MOST];
+#pragma unroll
+    for (int k = 0; k < 2 * Q3_TAPS_MOST; ++k)
+      if (k < 2 * taps && threadIdx.x + 64 * k < pieces) got[k] = src[threadIdx.x + 64 * k];
+#pragma unroll
+    for (int k = 0; k < 2 * Q3_TAPS_MOST; ++k)
+      if (k < 2 * taps && threadIdx.x + 64 * k < pieces) reinterpret_cast<float4*>(taps_of_block)[threadIdx.x + 64 * k] = got[k];
+  }
+  __syncthreads();
+  const int c0 = first + threadIdx.x * 8;
+  if (c0 >= C) return;
+  float tap[Q3_TAPS_MOST][8], base[8], add[8], win[Q3_TAPS_MOST - 1][8];
+  load8(bias + c0, base);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) add[e] = 0.f;
+  if (in_bias) load8(in_bias + c0, add);
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+#pragma unroll
+    for (int j = 0; j < Q3_TAPS_MOST; ++j)
+      tap[j][e] = j < taps ? taps_of_block[(threadIdx.x * 8 + e) * taps + taps - 1 - j] : 0.f;
+  }
+  const int t0 = blockIdx.x * rows_each;
+  const int t1 = t0 + rows_each < T ? t0 + rows_each : T;
+  if (rows_each == Q3_CONV_TILE && seq_index[t0] == seq_index[t1 - 1]) {
+    // the usual case, all rows of one sequence: every input the rows need is asked for at once (one wait
+    // instead of a chain of them), rows t0 - (taps - 1) .. t1 - 1 at in[Q3_TAPS_MOST - taps ..]
+    const int b = seq_index[t0];
+    const int start = cu[b];
+    const float* tail = state + (size_t)slots[b] * state_stride;
+    float in[Q3_CONV_TILE + Q3_TAPS_MOST - 1][8];
+#pragma unroll
+    for (int i = 0; i < Q3_CONV_TILE + Q3_TAPS_MOST - 1; ++i) {
+      const int row = t0 - (Q3_TAPS_MOST - 1) + i;
+      if (i >= Q3_TAPS_MOST - taps && row < t1) {
+        if (row >= start) {
+          load8(x + (size_t)row * x_stride + c0, in[i]);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) in[i][e] += add[e];
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) in[i][e] = tail[(size_t)(taps - 1 - (start - row)) * C + c0 + e];
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) in[i][e] = 0.f;
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < Q3_CONV_TILE; ++r) {
+      if (t0 + r < t1) {
+        float acc[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] = base[e];
+#pragma unroll
+        for (int j = 0; j < Q3_TAPS_MOST; ++j)
+          if (j < taps) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[e] += tap[j][e] * in[r + Q3_TAPS_MOST - 1 - j][e];
+          }
+        if (act == 1) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) acc[e] = silu_value(acc[e]);
+        }
+        store8(out + (size_t)(t0 + r) * C + c0, acc);
+      }
+    }
+    return;
+  }
+  for (int t = t0; t < t1; ++t) {
+    const int b = seq_index[t];
+    const int start = cu[b];
+    if (t == t0 || t == start) {
+      const float* tail = state + (size_t)slots[b] * state_stride;
+#pragma unroll
+      for (int j = 0; j < Q3_TAPS_MOST - 1; ++j) {
+        if (j < taps - 1) {
+          const int src = t - 1 - j;
+          if (src >= start) {
+            load8(x + (size_t)src * x_stride + c0, win[j]);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) win[j][e] += add[e];
+          } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) win[j][e] = tail[(size_t)(taps - 1 - (start - src)) * C + c0 + e];
+          }
+        }
+      }
+    }
+    float cur[8], acc[8];
+    load8(x + (size_t)t * x_stride + c0, cur);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      cur[e] += add[e];
+      acc[e] = base[e] + tap[0][e] * cur[e];
+    }
+#pragma unroll
+    for (int j = 0; j < Q3_TAPS_MOST - 1; ++j)
+      if (j < taps - 1) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] += tap[j + 1][e] * win[j][e];
+      }
+    if (act == 1) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) acc[e] = silu_value(acc[e]);
+    }
+    store8(out + (size_t)t * C + c0, acc);
+#pragma unroll
+    for (int j = Q3_TAPS_MOST - 2; j > 0; --j) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) win[j][e] = win[j - 1][e];
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) win[0][e] = cur[e];
+  }
+}
+
 // The tail after the step: the last taps - 1 inputs of the sequence, from this step's rows or,
 // for a step shorter than that, from the old tail moved up.
 template <typename TI>
@@ -439,36 +603,26 @@ __global__ void chunk_scan_kernel(float* __restrict__ sums, const float* __restr
   *mine = S;
 }
 
-// grid as chunk_state_kernel. A[t][s] = (q_t . k_s) exp(la_t - la_s) for s <= t, over d in slices of
-// 64 through shared memory; then o[t][j] = sum_s A[t][s] v_s[j] + exp(la_t) sum_i q_t[i] S[i][j] with
-// S the state before the chunk (from `sums`), again in slices of 64 over i.
-__global__ void __launch_bounds__(256) chunk_output_kernel(const float* __restrict__ q, const float* __restrict__ k,
-                                                           const float* __restrict__ v, const float* __restrict__ ld,
-                                                           long ld_row, const int* __restrict__ cu,
-                                                           const float* __restrict__ sums, float* __restrict__ out, int H,
-                                                           int hpg, int d, int dv) {
-  __shared__ float A[Q3_CHUNK * Q3_CHUNK];       // (t, s)
-  __shared__ float one[Q3_CHUNK * 65];           // a slice of q, rows padded to 65
-  __shared__ float two[Q3_CHUNK * 65];           // a slice of k (rows padded), then of S or v (rows of 64)
-  __shared__ float la[Q3_CHUNK];
-  const int b = blockIdx.z;
-  const int tiles = (dv + 63) / 64;
-  const int h = blockIdx.y / tiles, tile = blockIdx.y % tiles;
+// grid (chunks of the longest sequence, groups, B): the chunk's raw products q_t . k_s (64 x 64), over d in
+// slices of 64 through shared memory, into `scores` (chunk, group, t, s). They are the same for all heads of a
+// group and all tiles of a head's columns, which only weigh them with their own decays.
+__global__ void __launch_bounds__(256) chunk_scores_kernel(const float* __restrict__ q, const float* __restrict__ k,
+                                                           const int* __restrict__ cu, float* __restrict__ scores, int G,
+                                                           int d) {
+  __shared__ float one[Q3_CHUNK * 65];
+  __shared__ float two[Q3_CHUNK * 65];
+  const int b = blockIdx.z, g = blockIdx.y, c = blockIdx.x;
   const int start = cu[b], n = cu[b + 1] - start;
-  const int c = blockIdx.x;
   if (c * Q3_CHUNK >= n) return;
   const int row0 = start + c * Q3_CHUNK;
   const int len = n - c * Q3_CHUNK < Q3_CHUNK ? n - c * Q3_CHUNK : Q3_CHUNK;
   const int chunk = chunks_before(cu, b) + c;
-  const int G = H / hpg, g = h / hpg;
-  chunk_decays(la, ld, ld_row, h, row0, len);
-  const int tt = threadIdx.x / 16, tj = threadIdx.x % 16;      // rows tt + 16 r, columns 4 tj .. 4 tj + 3
+  const int tt = threadIdx.x / 16, tj = threadIdx.x % 16;
   float acc[4][4];
 #pragma unroll
   for (int r = 0; r < 4; ++r)
 #pragma unroll
     for (int x = 0; x < 4; ++x) acc[r][x] = 0.f;
-  // A = q k^T, a slice of 64 of d at a time
   for (int i0 = 0; i0 < d; i0 += 64) {
     __syncthreads();
     for (int e = threadIdx.x; e < Q3_CHUNK * 64; e += 256) {
@@ -490,14 +644,51 @@ __global__ void __launch_bounds__(256) chunk_output_kernel(const float* __restri
         for (int x = 0; x < 4; ++x) acc[r][x] += qv[r] * kv[x];
     }
   }
+  float* dst = scores + ((size_t)chunk * G + g) * Q3_CHUNK * Q3_CHUNK;
 #pragma unroll
   for (int r = 0; r < 4; ++r)
+    *reinterpret_cast<float4*>(dst + (tt + 16 * r) * Q3_CHUNK + 4 * tj) = make_float4(acc[r][0], acc[r][1], acc[r][2], acc[r][3]);
+}
+
+// grid as chunk_state_kernel. A[t][s] = scores[t][s] exp(la_t - la_s) for s <= t; then
+// o[t][j] = sum_s A[t][s] v_s[j] + exp(la_t) sum_i q_t[i] S[i][j] with S the state before the chunk (from `sums`),
+// in slices of 64 over i through shared memory.
+__global__ void __launch_bounds__(256) chunk_output_kernel(const float* __restrict__ q, const float* __restrict__ scores,
+                                                           const float* __restrict__ v, const float* __restrict__ ld,
+                                                           long ld_row, const int* __restrict__ cu,
+                                                           const float* __restrict__ sums, float* __restrict__ out, int H,
+                                                           int hpg, int d, int dv) {
+  __shared__ float A[Q3_CHUNK * Q3_CHUNK];       // (t, s)
+  __shared__ float one[Q3_CHUNK * 65];           // a slice of q, rows padded to 65
+  __shared__ float two[Q3_CHUNK * 64];           // a slice of S, then of v
+  __shared__ float la[Q3_CHUNK];
+  const int b = blockIdx.z;
+  const int tiles = (dv + 63) / 64;
+  const int h = blockIdx.y / tiles, tile = blockIdx.y % tiles;
+  const int start = cu[b], n = cu[b + 1] - start;
+  const int c = blockIdx.x;
+  if (c * Q3_CHUNK >= n) return;
+  const int row0 = start + c * Q3_CHUNK;
+  const int len = n - c * Q3_CHUNK < Q3_CHUNK ? n - c * Q3_CHUNK : Q3_CHUNK;
+  const int chunk = chunks_before(cu, b) + c;
+  const int G = H / hpg, g = h / hpg;
+  chunk_decays(la, ld, ld_row, h, row0, len);
+  __syncthreads();
+  const int tt = threadIdx.x / 16, tj = threadIdx.x % 16;      // rows tt + 16 r, columns 4 tj .. 4 tj + 3
+  float acc[4][4];
+  const float* raw = scores + ((size_t)chunk * G + g) * Q3_CHUNK * Q3_CHUNK;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int t = tt + 16 * r;
+    const float4 sc = *reinterpret_cast<const float4*>(raw + t * Q3_CHUNK + 4 * tj);
+    const float got[4] = {sc.x, sc.y, sc.z, sc.w};
 #pragma unroll
     for (int x = 0; x < 4; ++x) {
-      const int t = tt + 16 * r, s = 4 * tj + x;
-      A[t * Q3_CHUNK + s] = (s <= t && t < len) ? acc[r][x] * expf(la[t] - la[s]) : 0.f;
+      const int s = 4 * tj + x;
+      A[t * Q3_CHUNK + s] = (s <= t && t < len) ? got[x] * expf(la[t] - la[s]) : 0.f;
       acc[r][x] = 0.f;
     }
+  }
   // the state's share: exp(la_t) q_t S, a slice of 64 of d at a time
   const float* S = sums + ((size_t)chunk * H + h) * d * dv;
   for (int i0 = 0; i0 < d; i0 += 64) {
@@ -632,14 +823,14 @@ __global__ void retention_finish_kernel(const float* __restrict__ o, const TA* _
     out[(size_t)t * hv + h * vdim + j] = from_float<TA>(src[j] * inv * silu_value(to_float(gate[j])));
 }
 
-// Floats of workspace for a step of T rows in B sequences: q, k, v, ld, the chunks' sums and decays.
+// Floats of workspace for a step of T rows in B sequences: q, k, v, ld, the chunks' sums, decays and raw scores.
 extern "C" long q3_chunked_workspace(int T, int B, int H, int G, int d, int dv) {
   const long chunks = T / Q3_CHUNK + B;
-  return 2L * T * G * d + (long)T * H * dv + (long)T * H + chunks * H * ((long)d * dv + 1);
+  return 2L * T * G * d + (long)T * H * dv + (long)T * H + chunks * H * ((long)d * dv + 1) + chunks * G * Q3_CHUNK * Q3_CHUNK;
 }
 
 static int launch_chunks(const float* qf, const float* kf, const float* vf, const float* ld, long ld_row, float* sums,
-                         float* decays, float* state, long state_stride, const int* slots, const int* cu, float* out,
+                         float* decays, float* scores, float* state, long state_stride, const int* slots, const int* cu, float* out,
                          int B, int max_q_len, int H, int hpg, int d, int dv, hipStream_t stream) {
   const int chunks = (max_q_len + Q3_CHUNK - 1) / Q3_CHUNK;
   const int tiles = (dv + 63) / 64;
@@ -660,7 +851,8 @@ static int launch_chunks(const float* qf, const float* kf, const float* vf, cons
 #undef Q3_STATE
   hipLaunchKernelGGL(chunk_scan_kernel, dim3((d * dv + 255) / 256, H, B), dim3(256), 0, stream, sums, decays, state,
                      state_stride, slots, cu, H, d * dv);
-  hipLaunchKernelGGL(chunk_output_kernel, grid, dim3(256), 0, stream, qf, kf, vf, ld, ld_row, cu, sums, out, H, hpg, d,
+  hipLaunchKernelGGL(chunk_scores_kernel, dim3(chunks, H / hpg, B), dim3(256), 0, stream, qf, kf, cu, scores, H / hpg, d);
+  hipLaunchKernelGGL(chunk_output_kernel, grid, dim3(256), 0, stream, qf, scores, vf, ld, ld_row, cu, sums, out, H, hpg, d,
                      dv);
   return q3_launch_status();
 }
@@ -672,7 +864,8 @@ extern "C" int q3_mamba2_chunked(const void* xbc, const void* dt, long dt_stride
   if (T <= 0 || B <= 0 || H <= 0 || P <= 0 || N <= 0 || G <= 0 || H % G || max_q_len <= 0 || B > 65535)
     return Q3_ERR_BAD_ARGUMENT;
   if (N > 256 || (long)H * ((P + 63) / 64) > 65535) return Q3_ERR_UNSUPPORTED;
-  float* qf = workspace;
+  float* scores = workspace;        // first: it is read and written sixteen bytes at a time
+  float* qf = scores + (size_t)(T / Q3_CHUNK + B) * G * Q3_CHUNK * Q3_CHUNK;
   float* kf = qf + (size_t)T * G * N;
   float* vf = kf + (size_t)T * G * N;
   float* ld = vf + (size_t)T * H * P;
@@ -681,7 +874,7 @@ extern "C" int q3_mamba2_chunked(const void* xbc, const void* dt, long dt_stride
   Q3_DISPATCH_DTYPE(act_dtype, TA,
                     hipLaunchKernelGGL(mamba2_prepare_kernel<TA>, dim3(T), dim3(256), 0, stream, (const TA*)xbc,
                                        (const TA*)dt, dt_stride, dt_bias, a_log, qf, kf, vf, ld, H, P, N, G));
-  const int status = launch_chunks(qf, kf, vf, ld, H, sums, decays, state, state_stride, slots, cu, y, B, max_q_len, H,
+  const int status = launch_chunks(qf, kf, vf, ld, H, sums, decays, scores, state, state_stride, slots, cu, y, B, max_q_len, H,
                                    H / G, N, P, stream);
   if (status) return status;
   Q3_DISPATCH_DTYPE(act_dtype, TA,
@@ -700,7 +893,8 @@ extern "C" int q3_retention_chunked(const void* rows, const float* inv_freq, int
     return Q3_ERR_BAD_ARGUMENT;
   if (half > 0 && !inv_freq) return Q3_ERR_BAD_ARGUMENT;
   if (dim > 256 || (long)H * ((vdim + 63) / 64) > 65535) return Q3_ERR_UNSUPPORTED;
-  float* qf = workspace;
+  float* scores = workspace;
+  float* qf = scores + (size_t)(T / Q3_CHUNK + B) * H * Q3_CHUNK * Q3_CHUNK;
   float* kf = qf + (size_t)T * H * dim;
   float* vf = kf + (size_t)T * H * dim;
   float* ld = vf + (size_t)T * H * vdim;          // unused stretch: the decays are one number per head
@@ -709,7 +903,7 @@ extern "C" int q3_retention_chunked(const void* rows, const float* inv_freq, int
   Q3_DISPATCH_DTYPE(act_dtype, TA,
                     hipLaunchKernelGGL(retention_prepare_kernel<TA>, dim3(T), dim3(256), 0, stream, (const TA*)rows,
                                        inv_freq, half, positions, k_scale, qf, kf, vf, H, dim, vdim));
-  const int status = launch_chunks(qf, kf, vf, log_decays, 0, sums, decays, state, state_stride, slots, cu, scratch_out,
+  const int status = launch_chunks(qf, kf, vf, log_decays, 0, sums, decays, scores, state, state_stride, slots, cu, scratch_out,
                                    B, max_q_len, H, 1, dim, vdim, stream);
   if (status) return status;
   const int threads = vdim >= 256 ? 256 : (vdim >= 128 ? 128 : 64);
@@ -823,6 +1017,19 @@ extern "C" int q3_causal_conv(const void* x, long x_stride, const float* in_bias
   // `single_rows`: every sequence brings exactly one row (T == B); the tail then moves in the same kernel
   const bool fused = single_rows && T == B && taps > 1;
   const int rows_each = fused ? 1 : (T >= 2048 ? 16 : (T >= 256 ? 4 : 1));
+  const size_t in_size = in_dtype == Q3_F32 ? 4 : 2, out_size = out_dtype == Q3_F32 ? 4 : 2;
+  if (!fused && T >= 256 && C % 8 == 0 && x_stride % 8 == 0 && ((size_t)x % 16) == 0 && ((size_t)out % 16) == 0 &&
+      (x_stride * in_size) % 16 == 0 && (C * out_size) % 16 == 0 && ((size_t)bias % 16) == 0 && ((size_t)w % 16) == 0 &&
+      (!in_bias || ((size_t)in_bias % 16) == 0)) {
+    const int wide_threads = 64;       // the kernel's shared memory is sized for this
+    const int wide_rows = Q3_CONV_TILE;
+    Q3_DISPATCH_DTYPE(in_dtype, TI, Q3_DISPATCH_DTYPE(out_dtype, TO, {
+                        hipLaunchKernelGGL((causal_conv_wide_kernel<TI, TO>),
+                                           dim3((T + wide_rows - 1) / wide_rows, (C / 8 + wide_threads - 1) / wide_threads),
+                                           dim3(wide_threads), 0, stream, (const TI*)x, x_stride, in_bias, w, bias, state,
+                                           state_stride, slots, cu, seq_index, (TO*)out, T, C, taps, act, wide_rows);
+                      }));
+  } else
   Q3_DISPATCH_DTYPE(in_dtype, TI, Q3_DISPATCH_DTYPE(out_dtype, TO, {
                       hipLaunchKernelGGL((causal_conv_kernel<TI, TO>), dim3((T + rows_each - 1) / rows_each, chunks),
                                          dim3(threads), 0, stream, (const TI*)x, x_stride, in_bias, w, bias, state,

@@ -70,10 +70,11 @@ def test_hyper_norm(dtype, S, W):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("C,taps,lengths", [(70, 4, [1, 9, 2, 1]), (300, 3, [5, 1, 1, 40]), (64, 2, [3]), (33, 1, [2, 2]),
-                                            (80, 4, [1, 1, 1]), (40, 2, [1]), (96, 3, [300, 1, 20]), (64, 4, [2100, 3])])
+                                            (80, 4, [1, 1, 1]), (40, 2, [1]), (96, 3, [300, 1, 20]), (64, 4, [2100, 3]),
+                                            (4352, 4, [1, 2, 300, 1]), (72, 8, [3, 5, 250]), (100, 2, [260])])
 def test_causal_conv_continues_its_state(dtype, C, taps, lengths):
     g = _gen(C + taps)
-    wide = _rand(g, sum(lengths), C + 24, dtype=dtype)
+    wide = _rand(g, sum(lengths), C + (24 if C % 8 == 0 else 25), dtype=dtype)
     x = wide[:, 16:16 + C]
     weight, bias, add = _rand(g, C, taps), _rand(g, C), _rand(g, C)
     cu, seq, slots = _step(lengths, [4, 0, 2, 5][:len(lengths)])
