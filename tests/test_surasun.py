@@ -312,6 +312,27 @@ def test_greedy_generation_through_the_engine_on_the_host(cpu_ops, folder):
     assert engine.runner.manager.num_free() == 60
 
 
+def test_a_preempted_request_builds_its_state_again_on_the_host(cpu_ops, tmp_path):
+    """Too few pages for three requests at once: one is preempted, gives pages and state slot back, and
+    later goes through its prompt and its generated tokens again from an empty state. What it generates
+    is what it would have generated alone."""
+    folder = _write(tmp_path / "m", MIXED, peak=3.0)
+    config, w, _ = _truth(folder, {})
+    engine = SyncEngine(path=folder, dtype="float32", device="cpu", max_len=128, block_size=8, num_blocks=12,
+                        max_num_seqs=3, max_num_tokens=24, chunked_prefill_size=16)
+    prompts = [random_tokens(n, MIXED["vocab"], 300 + n) for n in (30, 9, 41)]
+    requests = [engine.add_request(p, engine.default_params(10, temperature=0.0, ignore_eos=True)) for p in prompts]
+    steps = 0
+    while engine.scheduler.has_work() and steps < 500:
+        engine.step()
+        engine.runner.manager.audit()
+        steps += 1
+    assert not engine.scheduler.has_work() and sum(r.preemptions for r in requests) >= 1
+    for prompt, request in zip(prompts, requests):
+        assert list(request.generated) == plain.greedy(config, w, prompt, 10)
+    assert engine.runner.manager.num_free() == 12
+
+
 def test_command_line_writes_a_folder_from_the_nested_config(tmp_path):
     from qwen3_from_scratch_amd.engine.cli import main
 
