@@ -119,6 +119,8 @@ class HyperConnectionBlock(Part):
     def __init__(self, prefix, precision, device, streams, mult=1.0):
         super().__init__(prefix, precision, device)
         self.streams, self.mult = int(streams), float(mult)
+        if not 0 <= self.streams <= 8:
+            raise ValueError("the kernel that updates and reads the streams takes up to 8 of them, not %d" % self.streams)
         self.mixer = self.feed_forward = self.mixer_norm = self.feed_forward_norm = None
         self.tables = {}
 

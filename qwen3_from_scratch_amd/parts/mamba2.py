@@ -27,6 +27,8 @@ class Mamba2(Part):
         super().__init__(prefix, precision, device)
         if heads % groups or (heads * vdim) % norm_groups:
             raise ValueError("groups must divide heads and norm_groups must divide heads * vdim")
+        if state > 256 or not 1 <= conv <= 8:
+            raise ValueError("the Mamba-2 kernels take a state of up to 256 and 1 to 8 taps, not %d and %d" % (state, conv))
         self.hidden_size, self.heads, self.vdim, self.state, self.groups = hidden_size, heads, vdim, state, groups
         self.taps, self.norm_groups, self.eps = conv, norm_groups, float(eps)
         self.inner = heads * vdim

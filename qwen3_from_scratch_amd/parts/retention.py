@@ -27,6 +27,9 @@ class Retention(Part):
         super().__init__(prefix, precision, device)
         if len(decay) != heads:
             raise ValueError("one decay per head: %d for %d heads" % (len(decay), heads))
+        if dim > 256 or rot_dims > dim or rot_dims % 2:
+            raise ValueError("retention's kernels take keys of up to 256 numbers and an even rotation within them, not %d and %d"
+                             % (dim, rot_dims))
         self.hidden_size, self.heads, self.dim, self.vdim = hidden_size, heads, dim, vdim
         self.decay_values, self.eps, self.rot_dims, self.rot_base = tuple(decay), float(eps), int(rot_dims), float(rot_base)
         self.w_in = self.w_out = self.decay = self.log_decay = self.inv_freq = None

@@ -28,6 +28,9 @@ class RecurrentUnit(Part):
         super().__init__(prefix, precision, device)
         if width % blocks:
             raise ValueError("blocks must divide width")
+        if width // blocks > 1536 or not 1 <= conv <= 8:
+            raise ValueError("the recurrent unit's kernels take blocks of up to 1,536 numbers and 1 to 8 taps, not %d and %d"
+                             % (width // blocks, conv))
         self.hidden_size, self.width, self.blocks, self.taps, self.rate = hidden_size, width, blocks, conv, float(rate)
         self.w_in = self.w_out = self.bias_y = self.bias_x = self.conv = self.conv_bias = None
         self.gate_weights = self.gate_biases = self.decay_rate = None

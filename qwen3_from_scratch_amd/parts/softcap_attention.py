@@ -32,6 +32,9 @@ class SoftcapAttention(Part):
         super().__init__(prefix, precision, device)
         if heads % kv_heads:
             raise ValueError("heads (%d) must be a multiple of kv_heads (%d)" % (heads, kv_heads))
+        if dim > 512 or vdim > 512 or rot_dims > dim or rot_dims % 2:
+            raise ValueError("the attention kernels take keys and values of up to 512 numbers and an even rotation within "
+                             "the keys, not %d, %d and %d" % (dim, vdim, rot_dims))
         self.hidden_size, self.heads, self.kv_heads, self.dim, self.vdim = hidden_size, heads, kv_heads, dim, vdim
         self.scale, self.eps, self.softcap, self.window = float(scale), float(eps), float(softcap), int(window)
         self.rot_dims, self.rot_base = int(rot_dims), float(rot_base)
