@@ -512,16 +512,17 @@ __device__ inline void chunk_decays(float* la, const float* __restrict__ ld, lon
 }
 
 // grid (chunks of the longest sequence, H * dv tiles of 64, B); 256 threads. U[i][j] = sum_s
-// exp(la_last - la_s) k_s[i] v_s[j] for the tile's 64 columns j, into `sums` (chunk, H, d, dv);
-// the chunk's whole decay exp(la_last) into `decays` (chunk, H).
-template <int DMAX>
+// exp(la_last - la_s) k_s[i] v_s[j] for the tile's 64 columns j, into `sums` (chunk, H, d, dv); the chunk's
+// whole decay exp(la_last) into `decays` (chunk, H). All threads bring k and v into shared memory; then eight
+// threads for every eight rows of d form 8 x 8 numbers each from 16-byte reads, four reads for 64 multiply-adds.
 __global__ void __launch_bounds__(256) chunk_state_kernel(const float* __restrict__ k, const float* __restrict__ v,
                                                           const float* __restrict__ ld, long ld_row,
                                                           const int* __restrict__ cu, float* __restrict__ sums,
                                                           float* __restrict__ decays, int H, int hpg, int d, int dv) {
-  extern __shared__ float lds[];
-  float* kw = lds;                          // (64, d)
-  float* vt = kw + Q3_CHUNK * d;            // (64, 64)
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  const int dp = (d + 7) / 8 * 8;           // rows of 8: the last ones may be zeros
+  float* kw = lds;                          // (64, dp)
+  float* vt = kw + Q3_CHUNK * dp;           // (64, 64)
   __shared__ float la[Q3_CHUNK];
   const int b = blockIdx.z;
   const int tiles = (dv + 63) / 64;
@@ -536,43 +537,63 @@ __global__ void __launch_bounds__(256) chunk_state_kernel(const float* __restric
   chunk_decays(la, ld, ld_row, h, row0, len);
   __syncthreads();
   const float last = la[len - 1];
-  for (int e = threadIdx.x; e < Q3_CHUNK * d; e += 256) {
-    const int s = e / d, i = e % d;
-    kw[e] = s < len ? k[((size_t)(row0 + s) * G + g) * d + i] * expf(last - la[s]) : 0.f;
-  }
-  for (int e = threadIdx.x; e < Q3_CHUNK * 64; e += 256) {
-    const int s = e / 64, j = tile * 64 + e % 64;
-    vt[e] = (s < len && j < dv) ? v[((size_t)(row0 + s) * H + h) * dv + j] : 0.f;
-  }
-  __syncthreads();
-  const int ti = threadIdx.x / 16, tj = threadIdx.x % 16;
-  float acc[DMAX / 16][4];
+  // sixteen loads a thread are asked for before the first is used (a loop of single loads is a chain of round trips)
+  for (int e0 = threadIdx.x; e0 < Q3_CHUNK * dp; e0 += 256 * 16) {
+    float got[16];
 #pragma unroll
-  for (int r = 0; r < DMAX / 16; ++r)
+    for (int u = 0; u < 16; ++u) {
+      const int e = e0 + 256 * u;
+      const int s = e / dp, i = e % dp;
+      got[u] = (e < Q3_CHUNK * dp && s < len && i < d) ? k[((size_t)(row0 + s) * G + g) * d + i] : 0.f;
+    }
 #pragma unroll
-    for (int x = 0; x < 4; ++x) acc[r][x] = 0.f;
-  for (int s = 0; s < len; ++s) {
-    const float4 vv = *reinterpret_cast<const float4*>(vt + s * 64 + 4 * tj);
-#pragma unroll
-    for (int r = 0; r < DMAX / 16; ++r) {
-      if (ti + 16 * r < d) {
-        const float kv = kw[s * d + ti + 16 * r];
-        acc[r][0] += kv * vv.x;
-        acc[r][1] += kv * vv.y;
-        acc[r][2] += kv * vv.z;
-        acc[r][3] += kv * vv.w;
-      }
+    for (int u = 0; u < 16; ++u) {
+      const int e = e0 + 256 * u;
+      if (e < Q3_CHUNK * dp) kw[e] = e / dp < len ? got[u] * expf(last - la[e / dp]) : 0.f;
     }
   }
-  float* dst = sums + ((size_t)chunk * H + h) * d * dv;
+  {
+    float got[16];
 #pragma unroll
-  for (int r = 0; r < DMAX / 16; ++r) {
-    const int i = ti + 16 * r;
-    if (i < d) {
+    for (int u = 0; u < 16; ++u) {
+      const int e = threadIdx.x + 256 * u;
+      const int s = e / 64, j = tile * 64 + e % 64;
+      got[u] = (s < len && j < dv) ? v[((size_t)(row0 + s) * H + h) * dv + j] : 0.f;
+    }
 #pragma unroll
-      for (int x = 0; x < 4; ++x) {
-        const int j = tile * 64 + 4 * tj + x;
-        if (j < dv) dst[(size_t)i * dv + j] = acc[r][x];
+    for (int u = 0; u < 16; ++u) vt[threadIdx.x + 256 * u] = got[u];
+  }
+  __syncthreads();
+  // (d up to 256: 32 groups of eight rows, eight threads each)
+  const int ti = threadIdx.x / 8, tj = threadIdx.x % 8;      // rows 8 ti .., columns 8 tj ..
+  if (8 * ti < dp) {
+    float acc[8][8];
+#pragma unroll
+    for (int r = 0; r < 8; ++r)
+#pragma unroll
+      for (int x = 0; x < 8; ++x) acc[r][x] = 0.f;
+    for (int s = 0; s < len; ++s) {
+      const float4 k0 = *reinterpret_cast<const float4*>(kw + s * dp + 8 * ti);
+      const float4 k1 = *reinterpret_cast<const float4*>(kw + s * dp + 8 * ti + 4);
+      const float4 v0 = *reinterpret_cast<const float4*>(vt + s * 64 + 8 * tj);
+      const float4 v1 = *reinterpret_cast<const float4*>(vt + s * 64 + 8 * tj + 4);
+      const float kk[8] = {k0.x, k0.y, k0.z, k0.w, k1.x, k1.y, k1.z, k1.w};
+      const float vv[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+#pragma unroll
+      for (int r = 0; r < 8; ++r)
+#pragma unroll
+        for (int x = 0; x < 8; ++x) acc[r][x] += kk[r] * vv[x];
+    }
+    float* dst = sums + ((size_t)chunk * H + h) * d * dv;
+#pragma unroll
+    for (int r = 0; r < 8; ++r) {
+      const int i = 8 * ti + r;
+      if (i < d) {
+#pragma unroll
+        for (int x = 0; x < 8; ++x) {
+          const int j = tile * 64 + 8 * tj + x;
+          if (j < dv) dst[(size_t)i * dv + j] = acc[r][x];
+        }
       }
     }
   }
@@ -625,11 +646,22 @@ __global__ void __launch_bounds__(256) chunk_scores_kernel(const float* __restri
     for (int x = 0; x < 4; ++x) acc[r][x] = 0.f;
   for (int i0 = 0; i0 < d; i0 += 64) {
     __syncthreads();
-    for (int e = threadIdx.x; e < Q3_CHUNK * 64; e += 256) {
-      const int s = e / 64, i = i0 + e % 64;
-      const bool in = s < len && i < d;
-      one[s * 65 + e % 64] = in ? q[((size_t)(row0 + s) * G + g) * d + i] : 0.f;
-      two[s * 65 + e % 64] = in ? k[((size_t)(row0 + s) * G + g) * d + i] : 0.f;
+    {
+      float gq[16], gk[16];
+#pragma unroll
+      for (int u = 0; u < 16; ++u) {
+        const int e = threadIdx.x + 256 * u;
+        const int s = e / 64, i = i0 + e % 64;
+        const bool in = s < len && i < d;
+        gq[u] = in ? q[((size_t)(row0 + s) * G + g) * d + i] : 0.f;
+        gk[u] = in ? k[((size_t)(row0 + s) * G + g) * d + i] : 0.f;
+      }
+#pragma unroll
+      for (int u = 0; u < 16; ++u) {
+        const int e = threadIdx.x + 256 * u;
+        one[(e / 64) * 65 + e % 64] = gq[u];
+        two[(e / 64) * 65 + e % 64] = gk[u];
+      }
     }
     __syncthreads();
     for (int i = 0; i < 64; ++i) {
@@ -693,11 +725,22 @@ __global__ void __launch_bounds__(256) chunk_output_kernel(const float* __restri
   const float* S = sums + ((size_t)chunk * H + h) * d * dv;
   for (int i0 = 0; i0 < d; i0 += 64) {
     __syncthreads();
-    for (int e = threadIdx.x; e < Q3_CHUNK * 64; e += 256) {
-      const int s = e / 64, i = i0 + e % 64;
-      one[s * 65 + e % 64] = (s < len && i < d) ? q[((size_t)(row0 + s) * G + g) * d + i] : 0.f;
-      const int si = i0 + e / 64, j = tile * 64 + e % 64;
-      two[e] = (si < d && j < dv) ? S[(size_t)si * dv + j] : 0.f;
+    {
+      float gq[16], gs[16];
+#pragma unroll
+      for (int u = 0; u < 16; ++u) {
+        const int e = threadIdx.x + 256 * u;
+        const int s = e / 64, i = i0 + e % 64;
+        gq[u] = (s < len && i < d) ? q[((size_t)(row0 + s) * G + g) * d + i] : 0.f;
+        const int si = i0 + e / 64, j = tile * 64 + e % 64;
+        gs[u] = (si < d && j < dv) ? S[(size_t)si * dv + j] : 0.f;
+      }
+#pragma unroll
+      for (int u = 0; u < 16; ++u) {
+        const int e = threadIdx.x + 256 * u;
+        one[(e / 64) * 65 + e % 64] = gq[u];
+        two[e] = gs[u];
+      }
     }
     __syncthreads();
     for (int i = 0; i < 64; ++i) {
@@ -720,9 +763,16 @@ __global__ void __launch_bounds__(256) chunk_output_kernel(const float* __restri
   }
   // the chunk's own share: A v
   __syncthreads();
-  for (int e = threadIdx.x; e < Q3_CHUNK * 64; e += 256) {
-    const int s = e / 64, j = tile * 64 + e % 64;
-    two[e] = (s < len && j < dv) ? v[((size_t)(row0 + s) * H + h) * dv + j] : 0.f;
+  {
+    float gv[16];
+#pragma unroll
+    for (int u = 0; u < 16; ++u) {
+      const int e = threadIdx.x + 256 * u;
+      const int s = e / 64, j = tile * 64 + e % 64;
+      gv[u] = (s < len && j < dv) ? v[((size_t)(row0 + s) * H + h) * dv + j] : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < 16; ++u) two[threadIdx.x + 256 * u] = gv[u];
   }
   __syncthreads();
   for (int s = 0; s < len; ++s) {
@@ -835,20 +885,16 @@ static int launch_chunks(const float* qf, const float* kf, const float* vf, cons
   const int chunks = (max_q_len + Q3_CHUNK - 1) / Q3_CHUNK;
   const int tiles = (dv + 63) / 64;
   const dim3 grid(chunks, H * tiles, B);
-  const size_t lds = (size_t)(Q3_CHUNK * d + Q3_CHUNK * 64) * sizeof(float);
-#define Q3_STATE(DMAX)                                                                                           \
-  hipLaunchKernelGGL(chunk_state_kernel<DMAX>, grid, dim3(256), lds, stream, kf, vf, ld, ld_row, cu, sums, decays, H, \
-                     hpg, d, dv)
-  if (d <= 64) Q3_STATE(64);
-  else if (d <= 128) Q3_STATE(128);
-  else {
-    // 64 rows of more than 128 numbers and the values' tile pass the 64 KB a launch may ask for unasked
-    const hipError_t allowed = hipFuncSetAttribute(reinterpret_cast<const void*>(chunk_state_kernel<256>),
+  const int dp = (d + 7) / 8 * 8;
+  const size_t lds = (size_t)(Q3_CHUNK * dp + Q3_CHUNK * 64) * sizeof(float);
+  if (lds > 64 * 1024) {
+    // 64 rows of more than 192 numbers and the values' tile pass the 64 KB a launch may ask for unasked
+    const hipError_t allowed = hipFuncSetAttribute(reinterpret_cast<const void*>(chunk_state_kernel),
                                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (allowed != hipSuccess) return (int)allowed;
-    Q3_STATE(256);
   }
-#undef Q3_STATE
+  hipLaunchKernelGGL(chunk_state_kernel, grid, dim3(256), lds, stream, kf, vf, ld, ld_row, cu, sums, decays, H, hpg, d,
+                     dv);
   hipLaunchKernelGGL(chunk_scan_kernel, dim3((d * dv + 255) / 256, H, B), dim3(256), 0, stream, sums, decays, state,
                      state_stride, slots, cu, H, d * dv);
   hipLaunchKernelGGL(chunk_scores_kernel, dim3(chunks, H / hpg, B), dim3(256), 0, stream, qf, kf, cu, scores, H / hpg, d);
