@@ -303,34 +303,67 @@ __global__ void __launch_bounds__(64) mamba2_scan_kernel(
 
 // ---- the recurrent unit's gates ----
 // out[g, t, b * bw + o] = sigmoid(bias[g, b, o] + sum_i w[g, b, i, o] * u[t, b * bw + i]) for the
-// two gates g, block-diagonal over `blocks` parts of bw numbers. A block of threads takes eight
-// tokens of one part of one gate; their u lie in shared memory.
+// two gates g, block-diagonal over `blocks` parts of bw numbers. A block of threads forms 64 tokens
+// by 64 outputs of one part and gate, over the inputs in slices of 64 that go through shared
+// memory (asked for in batches, as everywhere here); a thread holds 4 x 4 of them.
 #define Q3_GATE_TOKENS 8
-__global__ void block_gates_kernel(const float* __restrict__ u, const float* __restrict__ w,
-                                   const float* __restrict__ bias, float* __restrict__ out, int T, int width, int bw) {
-  extern __shared__ float su[];          // (Q3_GATE_TOKENS, bw)
-  const int t0 = blockIdx.x * Q3_GATE_TOKENS;
-  const int b = blockIdx.y, g = blockIdx.z;
+__global__ void __launch_bounds__(256) block_gates_kernel(const float* __restrict__ u, const float* __restrict__ w,
+                                                          const float* __restrict__ bias, float* __restrict__ out, int T,
+                                                          int width, int bw, int out_tiles) {
+  __shared__ float one[64 * 65];           // (token, input), rows padded
+  __shared__ __attribute__((aligned(16))) float two[64 * 64];           // (input, output)
+  const int t0 = blockIdx.x * 64;
+  const int b = blockIdx.y / out_tiles, o0 = (blockIdx.y % out_tiles) * 64, g = blockIdx.z;
   const int blocks = width / bw;
-  for (int i = threadIdx.x; i < Q3_GATE_TOKENS * bw; i += blockDim.x) {
-    const int tt = i / bw, e = i % bw;
-    su[i] = t0 + tt < T ? u[(size_t)(t0 + tt) * width + b * bw + e] : 0.f;
-  }
-  __syncthreads();
   const float* wb = w + ((size_t)g * blocks + b) * bw * bw;
-  for (int o = threadIdx.x; o < bw; o += blockDim.x) {
-    float acc[Q3_GATE_TOKENS];
-    const float start = bias[((size_t)g * blocks + b) * bw + o];
+  const int tt = threadIdx.x / 16, tj = threadIdx.x % 16;      // tokens tt + 16 r, outputs 4 tj .. 4 tj + 3
+  float acc[4][4];
 #pragma unroll
-    for (int tt = 0; tt < Q3_GATE_TOKENS; ++tt) acc[tt] = start;
-    for (int i = 0; i < bw; ++i) {
-      const float wv = wb[(size_t)i * bw + o];
+  for (int r = 0; r < 4; ++r)
 #pragma unroll
-      for (int tt = 0; tt < Q3_GATE_TOKENS; ++tt) acc[tt] += wv * su[tt * bw + i];
+    for (int x = 0; x < 4; ++x) acc[r][x] = 0.f;
+  for (int i0 = 0; i0 < bw; i0 += 64) {
+    __syncthreads();
+    {
+      float gu[16], gw[16];
+#pragma unroll
+      for (int k = 0; k < 16; ++k) {
+        const int e = threadIdx.x + 256 * k;
+        const int s = e / 64, c = e % 64;
+        gu[k] = (t0 + s < T && i0 + c < bw) ? u[(size_t)(t0 + s) * width + b * bw + i0 + c] : 0.f;
+        gw[k] = (i0 + s < bw && o0 + c < bw) ? wb[(size_t)(i0 + s) * bw + o0 + c] : 0.f;
+      }
+#pragma unroll
+      for (int k = 0; k < 16; ++k) {
+        const int e = threadIdx.x + 256 * k;
+        one[(e / 64) * 65 + e % 64] = gu[k];
+        two[e] = gw[k];
+      }
     }
+    __syncthreads();
+    for (int i = 0; i < 64; ++i) {
+      const float4 wv = *reinterpret_cast<const float4*>(two + i * 64 + 4 * tj);
 #pragma unroll
-    for (int tt = 0; tt < Q3_GATE_TOKENS; ++tt)
-      if (t0 + tt < T) out[((size_t)g * T + t0 + tt) * width + b * bw + o] = sigmoid_value(acc[tt]);
+      for (int r = 0; r < 4; ++r) {
+        const float uv = one[(tt + 16 * r) * 65 + i];
+        acc[r][0] += uv * wv.x;
+        acc[r][1] += uv * wv.y;
+        acc[r][2] += uv * wv.z;
+        acc[r][3] += uv * wv.w;
+      }
+    }
+  }
+#pragma unroll
+  for (int x = 0; x < 4; ++x) {
+    const int o = o0 + 4 * tj + x;
+    if (o < bw) {
+      const float start = bias[((size_t)g * blocks + b) * bw + o];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int t = t0 + tt + 16 * r;
+        if (t < T) out[((size_t)g * T + t) * width + b * bw + o] = sigmoid_value(start + acc[r][x]);
+      }
+    }
   }
 }
 
@@ -806,14 +839,28 @@ __global__ void mamba2_prepare_kernel(const TA* __restrict__ xbc, const TA* __re
                                       const float* __restrict__ dt_bias, const float* __restrict__ a_log,
                                       float* __restrict__ qf, float* __restrict__ kf, float* __restrict__ vf,
                                       float* __restrict__ ld, int H, int P, int N, int G) {
+  extern __shared__ float step_of_head[];      // (H): a head's step is formed once, not once per column
   const int t = blockIdx.x;
   const int C = H * P + 2 * G * N;
   const TA* row = xbc + (size_t)t * C;
-  for (int e = threadIdx.x; e < H * P; e += blockDim.x) {
-    const int h = e / P;
+  for (int h = threadIdx.x; h < H; h += blockDim.x) {
     const float step = softplus_value(to_float(dt[(size_t)t * dt_stride + h]) + dt_bias[h]);
-    vf[(size_t)t * H * P + e] = step * to_float(row[e]);
-    if (e % P == 0) ld[(size_t)t * H + h] = -expf(a_log[h]) * step;
+    step_of_head[h] = step;
+    ld[(size_t)t * H + h] = -expf(a_log[h]) * step;
+  }
+  __syncthreads();
+  for (int e0 = threadIdx.x; e0 < H * P; e0 += blockDim.x * 8) {
+    float got[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int e = e0 + blockDim.x * u;
+      got[u] = e < H * P ? to_float(row[e]) : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int e = e0 + blockDim.x * u;
+      if (e < H * P) vf[(size_t)t * H * P + e] = step_of_head[e / P] * got[u];
+    }
   }
   for (int e = threadIdx.x; e < G * N; e += blockDim.x) {
     kf[(size_t)t * G * N + e] = to_float(row[H * P + e]);
@@ -918,7 +965,7 @@ extern "C" int q3_mamba2_chunked(const void* xbc, const void* dt, long dt_stride
   float* sums = ld + (size_t)T * H;
   float* decays = sums + (size_t)(T / Q3_CHUNK + B) * H * N * P;
   Q3_DISPATCH_DTYPE(act_dtype, TA,
-                    hipLaunchKernelGGL(mamba2_prepare_kernel<TA>, dim3(T), dim3(256), 0, stream, (const TA*)xbc,
+                    hipLaunchKernelGGL(mamba2_prepare_kernel<TA>, dim3(T), dim3(256), (size_t)H * sizeof(float), stream, (const TA*)xbc,
                                        (const TA*)dt, dt_stride, dt_bias, a_log, qf, kf, vf, ld, H, P, N, G));
   const int status = launch_chunks(qf, kf, vf, ld, H, sums, decays, scores, state, state_stride, slots, cu, y, B, max_q_len, H,
                                    H / G, N, P, stream);
@@ -978,10 +1025,20 @@ __global__ void rglru_segment_kernel(const float* __restrict__ u, const float* _
   const int last = first + (n - seg * Q3_CHUNK < Q3_CHUNK ? n - seg * Q3_CHUNK : Q3_CHUNK);
   const float k = rate[c];
   float S = 0.f, logs = 0.f;
-  for (int t = first; t < last; ++t) {
-    const size_t at = (size_t)t * width + c;
-    logs += -k * gates[at];
-    rglru_step(S, k, gates[at], gates[(size_t)T * width + at], u[at]);
+  for (int t = first; t < last; t += 8) {        // eight rows' inputs asked for at once
+    float r[8], gi[8], uu[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const size_t at = (size_t)(t + j < last ? t + j : t) * width + c;
+      r[j] = gates[at], gi[j] = gates[(size_t)T * width + at], uu[j] = u[at];
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      if (t + j < last) {
+        logs += -k * r[j];
+        rglru_step(S, k, r[j], gi[j], uu[j]);
+      }
+    }
   }
   const size_t to = (size_t)(chunks_before(cu, b) + seg) * width + c;
   seg_decay[to] = expf(logs);
@@ -1020,11 +1077,23 @@ __global__ void rglru_apply_kernel(const float* __restrict__ u, const float* __r
   const int last = first + (n - seg * Q3_CHUNK < Q3_CHUNK ? n - seg * Q3_CHUNK : Q3_CHUNK);
   const float k = rate[c], yb = y_bias[c];
   float S = seg_state[(size_t)(chunks_before(cu, b) + seg) * width + c];
-  for (int t = first; t < last; ++t) {
-    const size_t at = (size_t)t * width + c;
-    rglru_step(S, k, gates[at], gates[(size_t)T * width + at], u[at]);
-    const float z = y[(size_t)t * y_stride + c] + yb;
-    out[at] = from_float<TO>(S * (0.5f * z * (1.f + tanhf(0.79788456080286536f * (z + 0.044715f * z * z * z)))));
+  for (int t = first; t < last; t += 8) {
+    float r[8], gi[8], uu[8], yy[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int row = t + j < last ? t + j : t;
+      const size_t at = (size_t)row * width + c;
+      r[j] = gates[at], gi[j] = gates[(size_t)T * width + at], uu[j] = u[at], yy[j] = y[(size_t)row * y_stride + c];
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      if (t + j < last) {
+        rglru_step(S, k, r[j], gi[j], uu[j]);
+        const float z = yy[j] + yb;
+        out[(size_t)(t + j) * width + c] =
+            from_float<TO>(S * (0.5f * z * (1.f + tanhf(0.79788456080286536f * (z + 0.044715f * z * z * z)))));
+      }
+    }
   }
 }
 
@@ -1121,7 +1190,7 @@ extern "C" int q3_block_gates(const float* u, const float* w, const float* bias,
   if (T <= 0 || width <= 0 || blocks <= 0 || width % blocks || blocks > 65535) return Q3_ERR_BAD_ARGUMENT;
   const int bw = width / blocks;
   if (bw > 1536) return Q3_ERR_UNSUPPORTED;
-  if (T <= 256) {
+  if (T <= 96) {
     const int out_tiles = (bw + 63) / 64;
     if ((long)blocks * out_tiles > 65535) return Q3_ERR_UNSUPPORTED;
     hipLaunchKernelGGL(block_gates_few_kernel, dim3((T + Q3_GATE_TOKENS - 1) / Q3_GATE_TOKENS, blocks * out_tiles, 2),
@@ -1129,9 +1198,10 @@ extern "C" int q3_block_gates(const float* u, const float* w, const float* bias,
                        bias, out, T, width, bw, out_tiles);
     return q3_launch_status();
   }
-  const int threads = bw >= 256 ? 256 : (bw >= 128 ? 128 : 64);
-  hipLaunchKernelGGL(block_gates_kernel, dim3((T + Q3_GATE_TOKENS - 1) / Q3_GATE_TOKENS, blocks, 2), dim3(threads),
-                     (size_t)Q3_GATE_TOKENS * bw * sizeof(float), stream, u, w, bias, out, T, width, bw);
+  const int out_tiles = (bw + 63) / 64;
+  if ((long)blocks * out_tiles > 65535) return Q3_ERR_UNSUPPORTED;
+  hipLaunchKernelGGL(block_gates_kernel, dim3((T + 63) / 64, blocks * out_tiles, 2), dim3(256), 0, stream, u, w, bias, out,
+                     T, width, bw, out_tiles);
   return q3_launch_status();
 }
 
