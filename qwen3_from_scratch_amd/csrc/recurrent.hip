@@ -112,7 +112,7 @@ __global__ void __launch_bounds__(64) causal_conv_wide_kernel(const TI* __restri
     float4 got[2 * Q3_TAPS_MOST];
 #pragma unroll
     for (int k = 0; k < 2 * Q3_TAPS_MOST; ++k)
-      if (k < 2 * taps && threadIdx.x + 64 * k < pieces) got[k] = src[threadIdx.x + 64 * k];
+      got[k] = (k < 2 * taps && threadIdx.x + 64 * k < pieces) ? src[threadIdx.x + 64 * k] : make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
     for (int k = 0; k < 2 * Q3_TAPS_MOST; ++k)
       if (k < 2 * taps && threadIdx.x + 64 * k < pieces) reinterpret_cast<float4*>(taps_of_block)[threadIdx.x + 64 * k] = got[k];
